@@ -1,0 +1,127 @@
+// Scatter of recomputed K/V rows into the paged cache, and block-table -> slot
+// expansion (gfx950).
+//
+// A token record is H_kv*D contiguous elements; it is moved as 16-byte chunks,
+// consecutive lanes on consecutive chunks, so a 1 KiB Dream record (H_kv = 4,
+// D = 128, bf16) is one wave64 store and an 8 KiB LLaDA record is two blocks'
+// worth of fully coalesced stores.  All layers go in one launch (grid.y).
+// HBM traffic per row and layer: 2 (K,V) * 2 (read+write) * H_kv * D * bytes.
+#include "common.h"
+
+namespace acache {
+
+struct ScatterParams {
+  char *k_cache;
+  char *v_cache;
+  const char *key;
+  const char *value;
+  const int32_t *slot_map;
+  int64_t N;
+  int64_t num_slots;
+  int64_t key_token_bytes;
+  int64_t value_token_bytes;
+  int64_t src_layer_bytes;
+  int64_t cache_layer_bytes;
+  int32_t chunks_per_token;  // H_kv * D * bytes / 16
+  int32_t L;
+};
+
+template <int LPB>
+__global__ __launch_bounds__(256) void scatter_kernel(ScatterParams p) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t token = gid / p.chunks_per_token;
+  if (token >= p.N) return;
+  const int chunk = (int)(gid - token * p.chunks_per_token);
+  const int64_t slot = p.slot_map[token];
+  if (slot < 0 || slot >= p.num_slots) return;  // -1 = "do not store"
+  const int l0 = blockIdx.y * LPB;
+  const int64_t dst = slot * p.chunks_per_token * 16 + (int64_t)chunk * 16;
+  const int64_t ksrc = token * p.key_token_bytes + (int64_t)chunk * 16;
+  const int64_t vsrc = token * p.value_token_bytes + (int64_t)chunk * 16;
+  vec16 k[LPB], v[LPB];
+#pragma unroll
+  for (int i = 0; i < LPB; ++i) {
+    if (l0 + i < p.L) {
+      k[i] = load16_stream(p.key + (int64_t)(l0 + i) * p.src_layer_bytes + ksrc);
+      v[i] = load16_stream(p.value + (int64_t)(l0 + i) * p.src_layer_bytes + vsrc);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < LPB; ++i) {
+    if (l0 + i < p.L) {
+      store16(p.k_cache + (int64_t)(l0 + i) * p.cache_layer_bytes + dst, k[i]);
+      store16(p.v_cache + (int64_t)(l0 + i) * p.cache_layer_bytes + dst, v[i]);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void block_table_slots_kernel(
+    int32_t *out, const int32_t *tables, const int32_t *cu_k, int B, int max_blocks,
+    int block_size) {
+  const int b = blockIdx.y;
+  const int start = cu_k[b];
+  const int len = cu_k[b + 1] - start;
+  for (int n = blockIdx.x * 256 + threadIdx.x; n < len; n += gridDim.x * 256) {
+    const int blk = n / block_size;
+    // a request longer than its table is a caller bug; map it to slot -1
+    // (readers treat out-of-range slots as absent) instead of reading past it
+    const int id = blk < max_blocks ? tables[(int64_t)b * max_blocks + blk] : -1;
+    out[start + n] = id < 0 ? -1 : id * block_size + (n - blk * block_size);
+  }
+}
+
+}  // namespace acache
+
+using namespace acache;
+
+extern "C" int acache_kv_scatter(
+    void *k_cache, void *v_cache, const void *key, const void *value, const int32_t *slot_map,
+    int64_t N, int32_t L, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int64_t key_token_stride, int64_t value_token_stride, int64_t src_layer_stride,
+    int64_t cache_layer_stride, void *stream) {
+  const int es = dtype_bytes(dtype);
+  if (es == 0) return fail(ACACHE_E_DTYPE, "kv_scatter: unknown dtype %d", dtype);
+  if (N < 0 || L < 0 || H_kv <= 0 || D <= 0 || num_slots < 0)
+    return fail(ACACHE_E_SHAPE, "kv_scatter: negative size");
+  if (N == 0 || L == 0) return 0;
+  if (!k_cache || !v_cache || !key || !value || !slot_map)
+    return fail(ACACHE_E_NULL, "kv_scatter: NULL pointer");
+  const int64_t tok = (int64_t)H_kv * D;
+  if ((tok * es) % 16) return fail(ACACHE_E_SHAPE, "kv_scatter: H_kv*D*bytes must be a multiple of 16");
+  if (key_token_stride < tok || value_token_stride < tok)
+    return fail(ACACHE_E_SHAPE, "kv_scatter: token stride smaller than H_kv*D");
+  if (!aligned16(k_cache) || !aligned16(v_cache) || !aligned16(key) || !aligned16(value) ||
+      (key_token_stride * es) % 16 || (value_token_stride * es) % 16 ||
+      (L > 1 && ((src_layer_stride * es) % 16 || (cache_layer_stride * es) % 16)))
+    return fail(ACACHE_E_ALIGN, "kv_scatter: pointers and strides must be 16-byte aligned");
+  if (L > 1 && cache_layer_stride < num_slots * tok)
+    return fail(ACACHE_E_SHAPE, "kv_scatter: cache layer stride smaller than one layer");
+  ScatterParams p;
+  p.k_cache = (char *)k_cache; p.v_cache = (char *)v_cache;
+  p.key = (const char *)key; p.value = (const char *)value; p.slot_map = slot_map;
+  p.N = N; p.num_slots = num_slots;
+  p.key_token_bytes = key_token_stride * es; p.value_token_bytes = value_token_stride * es;
+  p.src_layer_bytes = src_layer_stride * es; p.cache_layer_bytes = cache_layer_stride * es;
+  p.chunks_per_token = (int32_t)(tok * es / 16); p.L = L;
+  const int64_t gx = (N * p.chunks_per_token + 255) / 256;
+  if (gx > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "kv_scatter: too many rows");
+  constexpr int LPB = 2;
+  dim3 grid((unsigned)gx, (unsigned)((L + LPB - 1) / LPB));
+  hipLaunchKernelGGL(scatter_kernel<LPB>, grid, dim3(256), 0, (hipStream_t)stream, p);
+  return launch_status("scatter_kernel");
+}
+
+extern "C" int acache_block_table_slots(
+    int32_t *out_slots, const int32_t *block_tables, const int32_t *cu_k, int32_t B,
+    int32_t max_blocks, int32_t block_size, int64_t total_k, void *stream) {
+  if (B < 0 || max_blocks < 0 || block_size <= 0 || total_k < 0)
+    return fail(ACACHE_E_SHAPE, "block_table_slots: bad size");
+  if (B == 0 || total_k == 0) return 0;
+  if (!out_slots || !block_tables || !cu_k) return fail(ACACHE_E_NULL, "block_table_slots: NULL pointer");
+  if (B > 65535) return fail(ACACHE_E_SHAPE, "block_table_slots: batch %d > 65535", B);
+  int64_t gx = (total_k / B + 255) / 256 + 1;
+  if (gx > 1024) gx = 1024;
+  hipLaunchKernelGGL(block_table_slots_kernel, dim3((unsigned)gx, (unsigned)B), dim3(256), 0,
+                     (hipStream_t)stream, out_slots, block_tables, cu_k, B, max_blocks, block_size);
+  return launch_status("block_table_slots_kernel");
+}

@@ -1,0 +1,216 @@
+/*
+ * libacache_hip — C ABI of the MI355X (gfx950) affix-KV reuse kernels.
+ *
+ * The reference (sands-lab/ACache) has no C ABI: its boundary for this path is a
+ * set of Python callables that launch Triton kernels.  Each entry point below
+ * replaces one of those launches; the citation names the reference callable
+ * (path relative to the reference tree) whose arithmetic it reproduces.
+ *
+ * Conventions shared by every entry point
+ *   - all data pointers are DEVICE pointers owned by the caller; nothing is
+ *     allocated, freed or retained by the library;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
+ *     default stream) and the call returns without synchronising;
+ *   - return value: 0 = enqueued; < 0 = argument error (ACACHE_E_*), nothing was
+ *     launched; > 0 = the hipError_t reported by the launch;
+ *   - acache_last_error() returns a thread-local, human readable description of
+ *     the most recent non-zero return on the calling thread;
+ *   - calls are re-entrant across distinct streams; no global mutable state;
+ *   - strides and offsets are counted in ELEMENTS of `dtype`, never bytes;
+ *   - slot = block_id * cache_block_size + offset_in_block: an index into the
+ *     cache viewed as [num_slots, H_kv, D] (per layer).
+ */
+#ifndef ACACHE_HIP_H
+#define ACACHE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ACACHE_ABI_VERSION 1
+
+/* element types of K/V/Q payloads */
+#define ACACHE_BF16 0
+#define ACACHE_F16  1
+#define ACACHE_F32  2
+
+/* argument errors */
+#define ACACHE_E_NULL      -1  /* a required pointer is NULL                         */
+#define ACACHE_E_DTYPE     -2  /* dtype not supported by this entry point            */
+#define ACACHE_E_SHAPE     -3  /* head_dim / head counts / sizes not supported       */
+#define ACACHE_E_RANGE     -4  /* slot range, shift or table rows out of range       */
+#define ACACHE_E_OVERLAP   -5  /* source and destination rows overlap                */
+#define ACACHE_E_ALIGN     -6  /* pointer or stride breaks the 16-byte alignment rule */
+#define ACACHE_E_MODE      -7  /* inconsistent relocation arguments                  */
+
+int acache_abi_version(void);
+const char *acache_last_error(void);
+
+/*
+ * Relocate + RoPE re-rotate + gather into the packed varlen layout.
+ *
+ *   for l < L, t < T, h < H_kv:
+ *     out_k[l, t, h, :] = rotate(k_cache[l, slot_map[t], h, :], delta[t])
+ *     out_v[l, t, h, :] =        v_cache[l, slot_map[t], h, :]
+ *   rotate(x, d) = x * cos[|d|] + rot_half(x) * sgn(d) * sin[|d|],
+ *   rot_half(x)  = cat(-x[D/2:], x[:D/2]); fp32 multiply, multiply, add (each
+ *   rounded, no fused multiply-add), one rounding to `dtype` on store.
+ *   Rows with delta[t] == 0 (or delta == NULL) are bit copies.
+ *
+ * This is the un-fused form of the reference's key-side relocation inside
+ * attention (nano-vdllm/model/acache_attention.py:475-497: gather by
+ * read_slot_map, rotate rows of shared slots by delta = n - slot with the
+ * sin sign rule of line 496) and of the dense-cache slice copy of the HF path
+ * (llada/generate_ACache.py:501-512).
+ *
+ * Out-of-range inputs never fault: a row whose slot is outside [0, num_slots)
+ * or whose |delta| >= rope_rows is written as zeros (K and V).
+ *
+ * rope_cos / rope_sin: fp32 [rope_rows, D] contiguous, may be NULL iff delta is NULL.
+ * cache_layer_stride / out_layer_stride: elements between consecutive layers.
+ * Token rows are contiguous: [.., H_kv, D] with strides (H_kv*D, D, 1).
+ */
+int acache_relocate_rope_gather(
+    void *out_k, void *out_v,
+    const void *k_cache, const void *v_cache,
+    const int32_t *slot_map, const int32_t *delta,
+    const float *rope_cos, const float *rope_sin,
+    int64_t T, int32_t L, int32_t H_kv, int32_t D, int32_t dtype,
+    int64_t num_slots, int32_t rope_rows,
+    int64_t cache_layer_stride, int64_t out_layer_stride,
+    void *stream);
+
+/*
+ * In-place materialisation of a relocated affix copy, all layers in one launch.
+ *
+ *   for l < L, t < affix_len, h < H_kv:
+ *     k_cache[l, dst_slot + t, h, :] = rotate(k_cache[l, t, h, :], affix_shift)
+ *     v_cache[l, dst_slot + t, h, :] =        v_cache[l, t, h, :]
+ *
+ * Replaces materialize_relocated_affix and its per-layer launch loop
+ * (nano-vdllm/model/acache_attention.py:6-128; caller
+ * nano-vdllm/model_runner.py:314-341).  [0, affix_len) and
+ * [dst_slot, dst_slot + affix_len) must not overlap (ACACHE_E_OVERLAP) and must
+ * lie inside [0, num_slots); |affix_shift| < rope_rows (ACACHE_E_RANGE).
+ */
+int acache_materialize_relocated_affix(
+    void *k_cache, void *v_cache,
+    const float *rope_cos, const float *rope_sin,
+    int64_t dst_slot, int64_t affix_len, int32_t affix_shift,
+    int32_t L, int32_t H_kv, int32_t D, int32_t dtype,
+    int64_t num_slots, int32_t rope_rows, int64_t cache_layer_stride,
+    void *stream);
+
+/*
+ * Scatter freshly computed K/V rows into the paged cache.
+ *
+ *   for l < L, i < N: if slot_map[i] != -1:
+ *     k_cache[l, slot_map[i], :, :] = key[l, i, :, :]   (same for value)
+ *
+ * Replaces store_kvcache / store_kvcache_kernel
+ * (nano-vdllm/model/attention.py:11-41), which the reference launches once per
+ * layer (L = 1 here reproduces that call).  Rows are bit copies.  A slot outside
+ * [-1, num_slots) is skipped like -1.  Duplicate slots inside one call are
+ * undefined (as in the reference).
+ * key_token_stride / value_token_stride: elements between consecutive tokens
+ * of the source (>= H_kv*D, the reference's key.stride(0)); src_layer_stride:
+ * elements between layers of the source (ignored when L == 1).
+ */
+int acache_kv_scatter(
+    void *k_cache, void *v_cache,
+    const void *key, const void *value,
+    const int32_t *slot_map,
+    int64_t N, int32_t L, int32_t H_kv, int32_t D, int32_t dtype,
+    int64_t num_slots,
+    int64_t key_token_stride, int64_t value_token_stride,
+    int64_t src_layer_stride, int64_t cache_layer_stride,
+    void *stream);
+
+/*
+ * Per-request top-k anchor selection over ragged fp32 influence scores.
+ *
+ *   request b owns scores[cu_affix[b] .. cu_affix[b+1]) and selects
+ *   K_b = cu_k[b+1] - cu_k[b] indices: the first K_b under the order
+ *   "higher score first, then lower index" (largest != 0) or
+ *   "lower score first, then lower index" (largest == 0); they are written
+ *   ASCENDING to out_idx[cu_k[b] .. cu_k[b+1]) with offsets[b] added
+ *   (offsets may be NULL).
+ *
+ * Replaces torch.topk(...).indices.sort() at
+ * nano-vdllm/model_runner.py:833-843, llada/generate_ACache.py:247-260 and
+ * dream/generate_ACache.py:367-373.  torch leaves the order of equal scores
+ * unspecified; this library fixes it to the lower index.  -0.0 equals +0.0;
+ * NaN ranks above +inf (torch.topk's convention).  K_b is clamped to the
+ * request's score count.  idx_bytes selects int32 (4) or int64 (8) output.
+ */
+int acache_topk_anchors(
+    void *out_idx, const float *scores,
+    const int32_t *cu_affix, const int32_t *cu_k, const int32_t *offsets,
+    int32_t largest, int32_t B, int32_t idx_bytes,
+    void *stream);
+
+/*
+ * Expand per-request block tables into a flat slot map.
+ *
+ *   out_slots[cu_k[b] + n] = block_tables[b, n / block_size] * block_size + n % block_size
+ *   for n < cu_k[b+1] - cu_k[b]
+ *
+ * The addressing rule of the reference's block-table attention kernels
+ * (nano-vdllm/model/acache_attention.py:194-196, 295-297) and of
+ * prepare_decoding (nano-vdllm/model_runner.py:1100-1110).  Table entries past
+ * a request's last block (-1 padding) are never read.
+ */
+int acache_block_table_slots(
+    int32_t *out_slots, const int32_t *block_tables, const int32_t *cu_k,
+    int32_t B, int32_t max_blocks, int32_t block_size, int64_t total_k,
+    void *stream);
+
+/*
+ * Bidirectional variable-length attention reading K/V through a slot map.
+ *
+ *   per request b, head h (kv head = h / (H / H_kv)):
+ *     K_b[n] = k_cache[slot_map[cu_k[b] + n], kv head],  V_b[n] likewise
+ *     out[cu_q[b] + m, h] = softmax_n(q[cu_q[b] + m, h] . K_b[n] * scale) . V_b
+ *   fp32 accumulation, probabilities rounded to `dtype` before the PV product,
+ *   output rounded to `dtype`.
+ *
+ * Relocation modes (selected exactly as the reference wrapper does,
+ * nano-vdllm/model/acache_attention.py:670-671):
+ *   plain      : shared_prefix_len == 0 or affix_shifts == NULL
+ *   key side   : affix_shifts != NULL, shared_kv_lens == NULL — rows with
+ *                slot < shared_prefix_len are rotated by delta = n - slot
+ *                (lines 480-497)
+ *   query side : affix_shifts and shared_kv_lens given — the first
+ *                shared_kv_lens[b] keys of request b are scored against
+ *                q' = round(q*cos[s] - rot_half(q)*sin[s]), s = affix_shifts[b]
+ *                (lines 399-469)
+ * Replaces acache_attention / _acache_attention_kernel (lines 337-514, 643-738);
+ * with a slot map from acache_block_table_slots it also replaces
+ * baseline_ragged_attention and baseline_decode_attention (lines 131-334,
+ * 525-640).  Unlike the reference, rows of requests with no keys are written
+ * as zeros instead of being left uninitialised, and no host synchronisation is
+ * needed: the grid is sized from total_q and B.
+ *
+ * Supported: D == 128 or 64, dtype bf16 or f16, H % H_kv == 0.
+ * q / out: [total_q, H, D] with given token and head strides (innermost 1).
+ * k_cache / v_cache: [num_slots, H_kv, D] with given slot and head strides.
+ */
+int acache_varlen_attn(
+    void *out, const void *q, const void *k_cache, const void *v_cache,
+    const int32_t *cu_q, const int32_t *cu_k, const int32_t *slot_map,
+    float scale,
+    int32_t shared_prefix_len, const int32_t *shared_kv_lens, const int32_t *affix_shifts,
+    const float *rope_cos, const float *rope_sin, int32_t rope_rows,
+    int32_t B, int64_t total_q, int64_t total_k,
+    int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int64_t q_token_stride, int64_t q_head_stride,
+    int64_t out_token_stride, int64_t out_head_stride,
+    int64_t kv_slot_stride, int64_t kv_head_stride,
+    void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ACACHE_HIP_H */
