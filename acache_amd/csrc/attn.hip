@@ -1,9 +1,487 @@
-// placeholder until the MFMA kernel lands: reports an error, launches nothing
+// Bidirectional varlen attention over slot-mapped K/V on gfx950 MFMA.
+//
+// Work decomposition
+//   workgroup = 4 waves; each wave owns WQ = 16*NQ16 consecutive queries of one
+//   (request, head); the workgroup owns BM = 4*WQ queries and walks the request's
+//   keys in tiles of BN = 64, staged through LDS and shared by the 4 waves.
+//
+// MFMA formulation (v_mfma_f32_16x16x32, 64-wide wavefronts)
+//   S^T = K Q^T   : A = K tile rows (LDS, row-major, padded pitch), B = Q (registers)
+//   O^T = V^T P^T : A = V^T (LDS, transposed + XOR-swizzled on the way in),
+//                   B = P^T, which is exactly the accumulator layout of S^T after
+//                   a bf16 pack — probabilities never leave registers.
+//   In both products a lane owns ONE query column, so the running max, the
+//   rescale factor and the running sum are per-lane scalars; the only cross-lane
+//   traffic of the softmax is two xor-shuffles per tile for the row maximum.
+//
+// K/V rows are fetched through the slot map (16 lanes x 16 B per 256-byte row),
+// optionally re-rotated on the key side, and prefetched into registers one tile
+// ahead of the MFMA work.  HBM traffic per call: K and V rows once per
+// (request, kv head) when query tiles of one head share an L2 (the block index
+// is remapped so that they land on the same XCD), Q once, O once.
 #include "common.h"
+
+namespace acache {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+enum { MODE_PLAIN = 0, MODE_KEY_SIDE = 1, MODE_QUERY_SIDE = 2 };
+
+struct AttnParams {
+  char *out;
+  const char *q;
+  const char *k_cache;
+  const char *v_cache;
+  const int32_t *cu_q;
+  const int32_t *cu_k;
+  const int32_t *slot_map;
+  const int32_t *shared_kv_lens;
+  const int32_t *affix_shifts;
+  const float *cos_tab;
+  const float *sin_tab;
+  float scale_log2e;
+  int32_t shared_prefix_len;
+  int32_t rope_rows;
+  int32_t B;
+  int32_t H;
+  int32_t H_kv;
+  int32_t num_tiles;  // upper bound on the number of BM-row query tiles
+  int64_t num_slots;
+  int64_t q_token_bytes, q_head_bytes;
+  int64_t o_token_bytes, o_head_bytes;
+  int64_t kv_slot_bytes, kv_head_bytes;
+};
+
+template <int DTYPE> struct Mma;
+template <> struct Mma<ACACHE_BF16> {
+  __device__ static __forceinline__ f32x4 run(const vec16 &a, const vec16 &b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    return f32_to_bf16(lo) | (f32_to_bf16(hi) << 16);
+  }
+};
+template <> struct Mma<ACACHE_F16> {
+  __device__ static __forceinline__ f32x4 run(const vec16 &a, const vec16 &b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    return f32_to_f16(lo) | (f32_to_f16(hi) << 16);
+  }
+};
+
+// Rotate the (lo, hi) 16-byte chunk pair of one row: elements d0..d0+7 and
+// d0+D/2..d0+D/2+7.  sign = +1: x*cos + rot_half(x)*sin (key side);
+// sign = -1: x*cos - rot_half(x)*sin (query side).  Rounded once to DTYPE.
+template <int DTYPE, int D>
+__device__ __forceinline__ void rotate_pair(vec16 &lo, vec16 &hi, const float *cos_row,
+                                            const float *sin_row, int d0, float sign) {
+  using E = Elem<DTYPE>;
+  float a[8], b[8], ya[8], yb[8];
+  E::unpack(lo, a);
+  E::unpack(hi, b);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float cl = cos_row[d0 + j], sl = sign * sin_row[d0 + j];
+    const float ch = cos_row[d0 + D / 2 + j], sh = sign * sin_row[d0 + D / 2 + j];
+    ya[j] = a[j] * cl + (-b[j]) * sl;
+    yb[j] = b[j] * ch + a[j] * sh;
+  }
+  lo = E::pack(ya);
+  hi = E::pack(yb);
+}
+
+template <int DTYPE, int D, int NQ16, int MODE>
+__global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
+  constexpr int BN = 64;
+  constexpr int WQ = 16 * NQ16;
+  constexpr int BM = 4 * WQ;
+  constexpr int KS = D / 32;            // k-slabs of the QK^T product
+  constexpr int NT = BN / 16;           // 16-row key tiles per BN
+  constexpr int DT = D / 16;            // 16-row d tiles of O^T
+  constexpr int NS = BN / 32;           // 32-key slabs of the PV product
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int CH = ROW_BYTES / 16;    // 16-byte chunks per row
+  constexpr int PP = CH / 2;            // chunk pairs per row (K loader)
+  constexpr int K_ROWS_PER_PASS = 256 / PP;
+  constexpr int K_PASSES = BN / K_ROWS_PER_PASS;
+  constexpr int KPITCH = ROW_BYTES + 16;
+  constexpr int V_THREADS = CH * (BN / 4);  // one thread per (chunk, 4-row group)
+  constexpr int VPITCH = BN * 2;            // bytes per V^T row (swizzled, unpadded)
+  using M = Mma<DTYPE>;
+
+  __shared__ __attribute__((aligned(16))) char lds_k[BN * KPITCH];
+  __shared__ __attribute__((aligned(16))) char lds_v[D * VPITCH];
+
+  // ---- which (request, query tile, head) is this workgroup? -----------------
+  const int per_xcd = gridDim.x >> 3;
+  const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int group = p.H / p.H_kv;
+  if (w >= p.num_tiles * p.H) return;
+  const int hg = w % group;
+  int tile = (w / group) % p.num_tiles;
+  const int kvh = w / (group * p.num_tiles);
+  const int head = kvh * group + hg;
+  int b = 0, q_begin = 0, q_len = 0;
+  for (; b < p.B; ++b) {
+    q_begin = p.cu_q[b];
+    q_len = p.cu_q[b + 1] - q_begin;
+    const int tiles_b = (q_len + BM - 1) / BM;
+    if (tile < tiles_b) break;
+    tile -= tiles_b;
+  }
+  if (b >= p.B) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 15, lg = lane >> 4;
+  const int kv_begin = p.cu_k[b];
+  const int kv_len = p.cu_k[b + 1] - kv_begin;
+  const int q_tile0 = tile * BM;                  // first query row of the workgroup
+  const int q_wave0 = q_tile0 + wave * WQ;        // first query row of this wave
+  int nq_valid = (q_len - q_wave0 + 15) / 16;     // live 16-row query tiles of this wave
+  nq_valid = nq_valid < 0 ? 0 : (nq_valid > NQ16 ? NQ16 : nq_valid);
+
+  char *out_base = p.out + (int64_t)q_begin * p.o_token_bytes + (int64_t)head * p.o_head_bytes;
+
+  if (kv_len <= 0) {  // no keys: defined output (zeros)
+    for (int r = tid / CH; r < BM; r += 256 / CH) {
+      const int qr = q_tile0 + r;
+      if (qr < q_len) store16(out_base + (int64_t)qr * p.o_token_bytes + (tid % CH) * 16, vec16{{0, 0, 0, 0}});
+    }
+    return;
+  }
+
+  int shared_len = 0, shift = 0;
+  if (MODE == MODE_QUERY_SIDE) {
+    shared_len = p.shared_kv_lens[b];
+    shared_len = shared_len < 0 ? 0 : (shared_len > kv_len ? kv_len : shared_len);
+    shift = p.affix_shifts[b];
+    if (shift < 0 || shift >= p.rope_rows) shift = 0;  // out-of-table shift: leave unrotated
+  }
+
+  // ---- Q fragments (B operand): lane holds Q[query li][32*ks + 8*lg .. +8] ---
+  vec16 qf[NQ16][KS];
+  vec16 qs[MODE == MODE_QUERY_SIDE ? NQ16 : 1][KS];  // rotated copy for shared keys
+  const char *q_base = p.q + (int64_t)q_begin * p.q_token_bytes + (int64_t)head * p.q_head_bytes;
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    const int qr = q_wave0 + qt * 16 + li;
+    const bool live = qr < q_len;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      qf[qt][ks] = live ? load16(q_base + (int64_t)qr * p.q_token_bytes + (32 * ks + 8 * lg) * 2)
+                        : vec16{{0, 0, 0, 0}};
+    }
+    if (MODE == MODE_QUERY_SIDE) {
+      const float *cr = p.cos_tab + (int64_t)shift * D;
+      const float *sr = p.sin_tab + (int64_t)shift * D;
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) {  // partner of d is d + D/2: slab ks + KS/2, same lane
+        vec16 lo = qf[qt][ks], hi = qf[qt][ks + KS / 2];
+        if (shift != 0) rotate_pair<DTYPE, D>(lo, hi, cr, sr, 32 * ks + 8 * lg, -1.0f);
+        qs[qt][ks] = lo;
+        qs[qt][ks + KS / 2] = hi;
+      }
+    }
+  }
+
+  // ---- loader state ------------------------------------------------------------
+  // K: thread -> (row kr + pass*K_ROWS_PER_PASS, chunk pair kc / kc + PP)
+  const int kr = tid / PP, kc = tid % PP;
+  // V: thread -> (chunk vc, rows 4*vrg .. 4*vrg+3); threads >= V_THREADS idle
+  const int vc = tid % CH, vrg = tid / CH;
+  const bool v_thread = tid < V_THREADS;
+  vec16 k_lo[K_PASSES], k_hi[K_PASSES], v_row[4];
+  const char *kc_base = p.k_cache + (int64_t)kvh * p.kv_head_bytes;
+  const char *vc_base = p.v_cache + (int64_t)kvh * p.kv_head_bytes;
+
+  auto fetch = [&](int n0, int n_end) {
+#pragma unroll
+    for (int ps = 0; ps < K_PASSES; ++ps) {
+      const int n = n0 + kr + ps * K_ROWS_PER_PASS;
+      k_lo[ps] = vec16{{0, 0, 0, 0}};
+      k_hi[ps] = k_lo[ps];
+      if (n < n_end) {
+        const int64_t slot = p.slot_map[kv_begin + n];
+        if (slot >= 0 && slot < p.num_slots) {
+          const char *src = kc_base + slot * p.kv_slot_bytes + kc * 16;
+          k_lo[ps] = load16(src);
+          k_hi[ps] = load16(src + ROW_BYTES / 2);
+          if (MODE == MODE_KEY_SIDE && slot < p.shared_prefix_len) {
+            const int delta = n - (int)slot;
+            const int ad = delta < 0 ? -delta : delta;
+            if (delta != 0 && ad < p.rope_rows)
+              rotate_pair<DTYPE, D>(k_lo[ps], k_hi[ps], p.cos_tab + (int64_t)ad * D,
+                                    p.sin_tab + (int64_t)ad * D, kc * 8, delta < 0 ? -1.0f : 1.0f);
+          }
+        }
+      }
+    }
+    if (v_thread) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int n = n0 + 4 * vrg + r;
+        v_row[r] = vec16{{0, 0, 0, 0}};
+        if (n < n_end) {
+          const int64_t slot = p.slot_map[kv_begin + n];
+          if (slot >= 0 && slot < p.num_slots) v_row[r] = load16(vc_base + slot * p.kv_slot_bytes + vc * 16);
+        }
+      }
+    }
+  };
+
+  auto stage = [&]() {
+#pragma unroll
+    for (int ps = 0; ps < K_PASSES; ++ps) {
+      char *dst = lds_k + (kr + ps * K_ROWS_PER_PASS) * KPITCH + kc * 16;
+      store16(dst, k_lo[ps]);
+      store16(dst + ROW_BYTES / 2, k_hi[ps]);
+    }
+    if (v_thread) {
+      // 4 rows x 8 elements -> 8 columns x 4 keys; key n sits at position
+      // 32*(n/32) + 8*((n%16)/4) + 4*((n%32)/16) + n%4 inside its V^T row, the
+      // order in which the S^T accumulator hands probabilities to the PV product
+      const int n4 = 4 * vrg;
+      const int chunk = 4 * (n4 >> 5) + ((n4 & 15) >> 2);
+      const int half = (n4 & 31) >> 4;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int d = 8 * vc + j;
+        const uint32_t w0 = v_row[0].w[j >> 1], w1 = v_row[1].w[j >> 1];
+        const uint32_t w2 = v_row[2].w[j >> 1], w3 = v_row[3].w[j >> 1];
+        uint2 val;
+        if (j & 1) {
+          val.x = (w0 >> 16) | (w1 & 0xffff0000u);
+          val.y = (w2 >> 16) | (w3 & 0xffff0000u);
+        } else {
+          val.x = (w0 & 0xffffu) | (w1 << 16);
+          val.y = (w2 & 0xffffu) | (w3 << 16);
+        }
+        const int swz = ((d >> 1) & 7) ^ ((d >> 4) & 7);
+        *reinterpret_cast<uint2 *>(lds_v + d * VPITCH + ((chunk ^ swz) << 4) + (half << 3)) = val;
+      }
+    }
+  };
+
+  // ---- running softmax state, one query column per lane -------------------------
+  float m_run[NQ16], l_run[NQ16];
+  f32x4 o_acc[NQ16][DT];
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    m_run[qt] = -INFINITY;
+    l_run[qt] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = f32x4{0, 0, 0, 0};
+  }
+
+  // tiles: first the shared range [0, shared_len) (query-side mode only), then the rest
+  const int tiles_a = (shared_len + BN - 1) / BN;
+  const int tiles_b = (kv_len - shared_len + BN - 1) / BN;
+  const int n_tiles = tiles_a + tiles_b;
+  auto tile_range = [&](int t, int &n0, int &n_end) {
+    if (t < tiles_a) { n0 = t * BN; n_end = shared_len; }
+    else { n0 = shared_len + (t - tiles_a) * BN; n_end = kv_len; }
+  };
+
+  int n0, n_end;
+  tile_range(0, n0, n_end);
+  fetch(n0, n_end);
+
+  const float c = p.scale_log2e;
+  for (int t = 0; t < n_tiles; ++t) {
+    tile_range(t, n0, n_end);
+    const int n_valid = n_end - n0;  // keys of this tile that exist (may exceed BN)
+    const bool shared_tile = MODE == MODE_QUERY_SIDE && t < tiles_a;
+    stage();
+    __syncthreads();
+    if (t + 1 < n_tiles) {
+      int m0, m_end;
+      tile_range(t + 1, m0, m_end);
+      fetch(m0, m_end);
+    }
+
+    // K fragments (A operand): lane holds K[16*nt + li][32*ks + 8*lg .. +8]
+    f32x4 s_acc[NQ16][NT];
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] = f32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const vec16 kf = load16(lds_k + (16 * nt + li) * KPITCH + (4 * ks + lg) * 16);
+#pragma unroll
+        for (int qt = 0; qt < NQ16; ++qt) {
+          if (qt < nq_valid) {
+            const vec16 &qv = (MODE == MODE_QUERY_SIDE && shared_tile) ? qs[MODE == MODE_QUERY_SIDE ? qt : 0][ks]
+                                                                       : qf[qt][ks];
+            s_acc[qt][nt] = M::run(kf, qv, s_acc[qt][nt]);
+          }
+        }
+      }
+    }
+
+    // online softmax; P^T packed straight into the B operand of the PV product
+    vec16 pf[NQ16][NS];
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) {
+      if (qt < nq_valid) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+            mx = fmaxf(mx, s_acc[qt][nt][i]);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run[qt], mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = exp2f((m_run[qt] - m_use) * c);
+        const float mc = m_use * c;
+        float sum = 0.0f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float e = exp2f(s_acc[qt][nt][i] * c - mc);
+            s_acc[qt][nt][i] = e;
+            sum += e;
+          }
+        l_run[qt] = l_run[qt] * alpha + sum;
+        m_run[qt] = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
+          pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
+          pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
+          pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
+        }
+      }
+    }
+
+    // O^T += V^T P^T ; lane reads V^T[16*dt + li][keys of slab s, group lg]
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int d = 16 * dt + li;
+      const int swz = ((d >> 1) & 7) ^ ((d >> 4) & 7);
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const vec16 vf = load16(lds_v + d * VPITCH + (((4 * s + lg) ^ swz) << 4));
+#pragma unroll
+        for (int qt = 0; qt < NQ16; ++qt)
+          if (qt < nq_valid) o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
+      }
+    }
+    __syncthreads();  // every wave is done with this tile before it is overwritten
+  }
+
+  // ---- epilogue: normalise and store O[query li][16*dt + 4*lg .. +4] ------------
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    if (qt < nq_valid) {
+      float l = l_run[qt];
+      l += __shfl_xor(l, 16);
+      l += __shfl_xor(l, 32);
+      const float inv = l > 0.0f ? 1.0f / l : 1.0f;
+      const int qr = q_wave0 + qt * 16 + li;
+      if (qr < q_len) {
+        char *dst = out_base + (int64_t)qr * p.o_token_bytes + 4 * lg * 2;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          uint2 val;
+          val.x = M::pack2(o_acc[qt][dt][0] * inv, o_acc[qt][dt][1] * inv);
+          val.y = M::pack2(o_acc[qt][dt][2] * inv, o_acc[qt][dt][3] * inv);
+          *reinterpret_cast<uint2 *>(dst + 16 * dt * 2) = val;
+        }
+      }
+    }
+  }
+}
+
+template <int DTYPE, int D, int NQ16>
+static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStream_t stream) {
+  AttnParams p = p0;
+  constexpr int BM = 64 * NQ16;
+  p.num_tiles = (int32_t)((total_q + BM - 1) / BM) + p.B;
+  int64_t blocks = (int64_t)p.num_tiles * p.H;
+  blocks = (blocks + 7) / 8 * 8;  // the XCD remap needs a multiple of 8
+  if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
+  dim3 grid((unsigned)blocks), block(256);
+  switch (mode) {
+    case MODE_PLAIN:
+      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_PLAIN>), grid, block, 0, stream, p);
+      break;
+    case MODE_KEY_SIDE:
+      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_KEY_SIDE>), grid, block, 0, stream, p);
+      break;
+    default:
+      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_QUERY_SIDE>), grid, block, 0, stream, p);
+      break;
+  }
+  return launch_status("varlen_attn_kernel");
+}
+
+}  // namespace acache
+
+using namespace acache;
+
 extern "C" int acache_varlen_attn(
-    void *, const void *, const void *, const void *, const int32_t *, const int32_t *, const int32_t *,
-    float, int32_t, const int32_t *, const int32_t *, const float *, const float *, int32_t,
-    int32_t, int64_t, int64_t, int32_t, int32_t, int32_t, int32_t, int64_t,
-    int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, void *) {
-  return acache::fail(ACACHE_E_MODE, "varlen_attn: kernel not built yet");
+    void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *cu_q,
+    const int32_t *cu_k, const int32_t *slot_map, float scale, int32_t shared_prefix_len,
+    const int32_t *shared_kv_lens, const int32_t *affix_shifts, const float *rope_cos,
+    const float *rope_sin, int32_t rope_rows, int32_t B, int64_t total_q, int64_t total_k, int32_t H,
+    int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t q_token_stride,
+    int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t kv_slot_stride,
+    int64_t kv_head_stride, void *stream) {
+  if (dtype != ACACHE_BF16 && dtype != ACACHE_F16)
+    return fail(ACACHE_E_DTYPE, "varlen_attn: dtype %d not supported (bf16 or f16)", dtype);
+  if (D != 128 && D != 64) return fail(ACACHE_E_SHAPE, "varlen_attn: head_dim %d not supported (64 or 128)", D);
+  if (B < 0 || total_q < 0 || total_k < 0 || H <= 0 || H_kv <= 0 || H % H_kv != 0 || num_slots < 0)
+    return fail(ACACHE_E_SHAPE, "varlen_attn: bad sizes (H=%d, H_kv=%d)", H, H_kv);
+  if (B == 0 || total_q == 0) return 0;
+  if (!out || !q || !cu_q || !cu_k) return fail(ACACHE_E_NULL, "varlen_attn: NULL pointer");
+  if (total_k > 0 && (!k_cache || !v_cache || !slot_map))
+    return fail(ACACHE_E_NULL, "varlen_attn: NULL cache or slot map");
+  const bool relocate = shared_prefix_len > 0 && affix_shifts != nullptr;
+  const bool query_side = relocate && shared_kv_lens != nullptr;
+  if (relocate && (!rope_cos || !rope_sin || rope_rows <= 0))
+    return fail(ACACHE_E_MODE, "varlen_attn: relocation requested without RoPE tables");
+  const int es = 2;
+  if (!aligned16(out) || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) ||
+      (q_token_stride * es) % 16 || (q_head_stride * es) % 16 || (out_token_stride * es) % 16 ||
+      (out_head_stride * es) % 16 || (kv_slot_stride * es) % 16 || (kv_head_stride * es) % 16)
+    return fail(ACACHE_E_ALIGN, "varlen_attn: pointers and strides must be 16-byte aligned");
+  AttnParams p;
+  p.out = (char *)out; p.q = (const char *)q;
+  p.k_cache = (const char *)k_cache; p.v_cache = (const char *)v_cache;
+  p.cu_q = cu_q; p.cu_k = cu_k; p.slot_map = slot_map;
+  p.shared_kv_lens = shared_kv_lens; p.affix_shifts = affix_shifts;
+  p.cos_tab = rope_cos; p.sin_tab = rope_sin;
+  p.scale_log2e = scale * 1.4426950408889634f;
+  p.shared_prefix_len = relocate ? shared_prefix_len : 0;
+  p.rope_rows = rope_rows; p.B = B; p.H = H; p.H_kv = H_kv; p.num_tiles = 0;
+  p.num_slots = num_slots;
+  p.q_token_bytes = q_token_stride * es; p.q_head_bytes = q_head_stride * es;
+  p.o_token_bytes = out_token_stride * es; p.o_head_bytes = out_head_stride * es;
+  p.kv_slot_bytes = kv_slot_stride * es; p.kv_head_bytes = kv_head_stride * es;
+  const int mode = query_side ? MODE_QUERY_SIDE : (relocate ? MODE_KEY_SIDE : MODE_PLAIN);
+  hipStream_t st = (hipStream_t)stream;
+#define ACACHE_ATTN(DT, DD) \
+  if (dtype == DT && D == DD) return launch_attn<DT, DD, 2>(p, mode, total_q, st);
+  ACACHE_ATTN(ACACHE_BF16, 128)
+  ACACHE_ATTN(ACACHE_BF16, 64)
+  ACACHE_ATTN(ACACHE_F16, 128)
+  ACACHE_ATTN(ACACHE_F16, 64)
+#undef ACACHE_ATTN
+  return fail(ACACHE_E_SHAPE, "varlen_attn: unsupported configuration");
 }
