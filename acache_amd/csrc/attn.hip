@@ -80,6 +80,10 @@ template <> struct Mma<ACACHE_F16> {
 template <int DTYPE, int D>
 __device__ __forceinline__ void rotate_pair(vec16 &lo, vec16 &hi, const float *cos_row,
                                             const float *sin_row, int d0, float sign) {
+  // products and sum rounded separately, exactly like the stand-alone relocation
+  // kernel, so key-side attention and attention over a materialised copy see
+  // bit-identical keys
+#pragma clang fp contract(off)
   using E = Elem<DTYPE>;
   float a[8], b[8], ya[8], yb[8];
   E::unpack(lo, a);
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
 
   // ---- Q fragments (B operand): lane holds Q[query li][32*ks + 8*lg .. +8] ---
   vec16 qf[NQ16][KS];
-  vec16 qs[MODE == MODE_QUERY_SIDE ? NQ16 : 1][KS];  // rotated copy for shared keys
+  vec16 qs[NQ16][KS];  // query-side mode: rotated copy scored against the shared keys
   const char *q_base = p.q + (int64_t)q_begin * p.q_token_bytes + (int64_t)head * p.q_head_bytes;
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
@@ -311,21 +315,20 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
     for (int qt = 0; qt < NQ16; ++qt)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] = f32x4{0, 0, 0, 0};
+    auto scores = [&](const vec16 (&qq)[NQ16][KS]) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
+      for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const vec16 kf = load16(lds_k + (16 * nt + li) * KPITCH + (4 * ks + lg) * 16);
+        for (int ks = 0; ks < KS; ++ks) {
+          const vec16 kf = load16(lds_k + (16 * nt + li) * KPITCH + (4 * ks + lg) * 16);
 #pragma unroll
-        for (int qt = 0; qt < NQ16; ++qt) {
-          if (qt < nq_valid) {
-            const vec16 &qv = (MODE == MODE_QUERY_SIDE && shared_tile) ? qs[MODE == MODE_QUERY_SIDE ? qt : 0][ks]
-                                                                       : qf[qt][ks];
-            s_acc[qt][nt] = M::run(kf, qv, s_acc[qt][nt]);
-          }
+          for (int qt = 0; qt < NQ16; ++qt)
+            if (qt < nq_valid) s_acc[qt][nt] = M::run(kf, qq[qt][ks], s_acc[qt][nt]);
         }
       }
-    }
+    };
+    if (MODE == MODE_QUERY_SIDE && shared_tile) scores(qs);
+    else scores(qf);
 
     // online softmax; P^T packed straight into the B operand of the PV product
     vec16 pf[NQ16][NS];
@@ -448,6 +451,8 @@ extern "C" int acache_varlen_attn(
   if (D != 128 && D != 64) return fail(ACACHE_E_SHAPE, "varlen_attn: head_dim %d not supported (64 or 128)", D);
   if (B < 0 || total_q < 0 || total_k < 0 || H <= 0 || H_kv <= 0 || H % H_kv != 0 || num_slots < 0)
     return fail(ACACHE_E_SHAPE, "varlen_attn: bad sizes (H=%d, H_kv=%d)", H, H_kv);
+  if (!(scale > 0.0f) || scale > 3.0e38f)
+    return fail(ACACHE_E_RANGE, "varlen_attn: softmax scale must be positive and finite");
   if (B == 0 || total_q == 0) return 0;
   if (!out || !q || !cu_q || !cu_k) return fail(ACACHE_E_NULL, "varlen_attn: NULL pointer");
   if (total_k > 0 && (!k_cache || !v_cache || !slot_map))

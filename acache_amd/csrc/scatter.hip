@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void block_table_slots_kernel(
   for (int n = blockIdx.x * 256 + threadIdx.x; n < len; n += gridDim.x * 256) {
     const int blk = n / block_size;
     // a request longer than its table is a caller bug; map it to slot -1
-    // (readers treat out-of-range slots as absent) instead of reading past it
+    // (readers turn out-of-range slots into zero rows) instead of reading past it
     const int id = blk < max_blocks ? tables[(int64_t)b * max_blocks + blk] : -1;
     out[start + n] = id < 0 ? -1 : id * block_size + (n - blk * block_size);
   }

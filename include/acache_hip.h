@@ -193,7 +193,8 @@ int acache_block_table_slots(
  * as zeros instead of being left uninitialised, and no host synchronisation is
  * needed: the grid is sized from total_q and B.
  *
- * Supported: D == 128 or 64, dtype bf16 or f16, H % H_kv == 0.
+ * Supported: D == 128 or 64, dtype bf16 or f16, H % H_kv == 0, scale > 0 (ACACHE_E_RANGE
+ * otherwise).  A key whose slot lies outside [0, num_slots) reads as a zero row.
  * q / out: [total_q, H, D] with given token and head strides (innermost 1).
  * k_cache / v_cache: [num_slots, H_kv, D] with given slot and head strides.
  */
