@@ -29,6 +29,11 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 enum { MODE_PLAIN = 0, MODE_KEY_SIDE = 1, MODE_QUERY_SIDE = 2 };
 
+// Source of absent rows for the global->LDS copies: a key past the end of its
+// range, or one whose slot lies outside the cache, is fetched from here, so the
+// LDS tiles are written by the copy engine only (no competing ds_write).
+__device__ __attribute__((aligned(256))) const uint32_t kZeroRow[64] = {0};
+
 struct AttnParams {
   char *out;
   const char *q;
@@ -99,8 +104,20 @@ __device__ __forceinline__ void rotate_pair(vec16 &lo, vec16 &hi, const float *c
   hi = E::pack(yb);
 }
 
+// Key range of tile t: the shared range [0, shared_len) comes first in tiles of BN
+// (query-side mode only, otherwise shared_len = 0), then [shared_len, kv_len).
+struct TileRange {
+  int n0, n_end;
+};
+__device__ __forceinline__ TileRange tile_range_of(int t, int tiles_a, int shared_len, int kv_len, int BN) {
+  TileRange r;
+  if (t < tiles_a) { r.n0 = t * BN; r.n_end = shared_len; }
+  else { r.n0 = shared_len + (t - tiles_a) * BN; r.n_end = kv_len; }
+  return r;
+}
+
 template <int DTYPE, int D, int NQ16, int MODE>
-__global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
   constexpr int BN = 64;
   constexpr int WQ = 16 * NQ16;
   constexpr int BM = 4 * WQ;
@@ -204,7 +221,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
   const char *kc_base = p.k_cache + (int64_t)kvh * p.kv_head_bytes;
   const char *vc_base = p.v_cache + (int64_t)kvh * p.kv_head_bytes;
 
-  auto fetch = [&](int n0, int n_end) {
+  auto fetch = [&](int n0, int n_end) __attribute__((always_inline)) {
 #pragma unroll
     for (int ps = 0; ps < K_PASSES; ++ps) {
       const int n = n0 + kr + ps * K_ROWS_PER_PASS;
@@ -239,7 +256,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
     }
   };
 
-  auto stage = [&]() {
+  auto stage = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int ps = 0; ps < K_PASSES; ++ps) {
       char *dst = lds_k + (kr + ps * K_ROWS_PER_PASS) * KPITCH + kc * 16;
@@ -287,35 +304,32 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
   const int tiles_a = (shared_len + BN - 1) / BN;
   const int tiles_b = (kv_len - shared_len + BN - 1) / BN;
   const int n_tiles = tiles_a + tiles_b;
-  auto tile_range = [&](int t, int &n0, int &n_end) {
-    if (t < tiles_a) { n0 = t * BN; n_end = shared_len; }
-    else { n0 = shared_len + (t - tiles_a) * BN; n_end = kv_len; }
-  };
 
   int n0, n_end;
-  tile_range(0, n0, n_end);
+  { const TileRange tr = tile_range_of(0, tiles_a, shared_len, kv_len, BN); n0 = tr.n0; n_end = tr.n_end; }
   fetch(n0, n_end);
 
   const float c = p.scale_log2e;
   for (int t = 0; t < n_tiles; ++t) {
-    tile_range(t, n0, n_end);
+    { const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN); n0 = tr.n0; n_end = tr.n_end; }
     const int n_valid = n_end - n0;  // keys of this tile that exist (may exceed BN)
     const bool shared_tile = MODE == MODE_QUERY_SIDE && t < tiles_a;
     stage();
     __syncthreads();
     if (t + 1 < n_tiles) {
       int m0, m_end;
-      tile_range(t + 1, m0, m_end);
+      { const TileRange tr = tile_range_of(t + 1, tiles_a, shared_len, kv_len, BN); m0 = tr.n0; m_end = tr.n_end; }
       fetch(m0, m_end);
     }
 
+    if (nq_valid > 0) {  // waves past the end of the request only help with the loads
     // K fragments (A operand): lane holds K[16*nt + li][32*ks + 8*lg .. +8]
     f32x4 s_acc[NQ16][NT];
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt)
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] = f32x4{0, 0, 0, 0};
-    auto scores = [&](const vec16 (&qq)[NQ16][KS]) {
+    auto scores = [&](const vec16 (&qq)[NQ16][KS]) __attribute__((always_inline)) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
@@ -323,7 +337,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
           const vec16 kf = load16(lds_k + (16 * nt + li) * KPITCH + (4 * ks + lg) * 16);
 #pragma unroll
           for (int qt = 0; qt < NQ16; ++qt)
-            if (qt < nq_valid) s_acc[qt][nt] = M::run(kf, qq[qt][ks], s_acc[qt][nt]);
+            s_acc[qt][nt] = M::run(kf, qq[qt][ks], s_acc[qt][nt]);
         }
       }
     };
@@ -334,7 +348,7 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
     vec16 pf[NQ16][NS];
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt) {
-      if (qt < nq_valid) {
+      {
         float mx = -INFINITY;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
@@ -382,13 +396,325 @@ __global__ __launch_bounds__(256) void varlen_attn_kernel(AttnParams p) {
         const vec16 vf = load16(lds_v + d * VPITCH + (((4 * s + lg) ^ swz) << 4));
 #pragma unroll
         for (int qt = 0; qt < NQ16; ++qt)
-          if (qt < nq_valid) o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
+          o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
       }
+    }
     }
     __syncthreads();  // every wave is done with this tile before it is overwritten
   }
 
   // ---- epilogue: normalise and store O[query li][16*dt + 4*lg .. +4] ------------
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    if (qt < nq_valid) {
+      float l = l_run[qt];
+      l += __shfl_xor(l, 16);
+      l += __shfl_xor(l, 32);
+      const float inv = l > 0.0f ? 1.0f / l : 1.0f;
+      const int qr = q_wave0 + qt * 16 + li;
+      if (qr < q_len) {
+        char *dst = out_base + (int64_t)qr * p.o_token_bytes + 4 * lg * 2;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          uint2 val;
+          val.x = M::pack2(o_acc[qt][dt][0] * inv, o_acc[qt][dt][1] * inv);
+          val.y = M::pack2(o_acc[qt][dt][2] * inv, o_acc[qt][dt][3] * inv);
+          *reinterpret_cast<uint2 *>(dst + 16 * dt * 2) = val;
+        }
+      }
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------
+// DMA variant (plain and query-side modes): K/V rows go global -> LDS directly
+// (global_load_lds, 16 B per lane, no staging registers) into a two-deep ring,
+// and V^T fragments are produced by the LDS transpose read ds_read_b64_tr_b16,
+// so V stays row-major and needs no register transpose.
+//
+// LDS tile layout: [BN rows][D*2 bytes], unpadded; the 16-byte chunk c of row r
+// sits at chunk position c ^ f(r).  The permutation is applied on the global
+// side (each lane fetches the chunk that belongs at its LDS position), so the
+// DMA writes stay linear.  f_K(r) = (r/RW) % CH makes the 16 rows of a K
+// fragment read (ds_read_b128) hit 16 different bank groups; f_V(r) =
+// 2*((r/RW) % (CH/2)) does the same for the 16 rows x 32 B of a transpose read.
+// RW = rows per 256-byte bank window, CH = chunks per row.
+//
+// ds_read_b64_tr_b16 within a 16-lane group: lane l supplies the address of
+// 4 consecutive 16-bit elements; lane i receives element i%4 of the lanes
+// 4*j + i/4, j = 0..3.  With lane l pointing at V[row0 + l/4][d0 + 4*(l%4)] lane i
+// gets V[row0 + 0..3][d0 + i]: four keys of one column, i.e. half of an MFMA
+// A-operand of V^T.
+template <int DTYPE, int D, int NQ16, int MODE>
+__global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
+  static_assert(MODE != MODE_KEY_SIDE, "key-side rotation needs the register-staged kernel");
+  constexpr int BN = 64;
+  constexpr int WQ = 16 * NQ16;
+  constexpr int BM = 4 * WQ;
+  constexpr int KS = D / 32;
+  constexpr int NT = BN / 16;
+  constexpr int DT = D / 16;
+  constexpr int NS = BN / 32;
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int CH = ROW_BYTES / 16;          // chunks per row: 16 (D=128) or 8 (D=64)
+  constexpr int RW = 256 / ROW_BYTES;         // rows per bank window: 1 or 2
+  constexpr int RPI = 64 / CH;                // rows per DMA instruction: 4 or 8
+  constexpr int WAVE_ROWS = BN / 4;           // 16 rows of every tile belong to each wave
+  constexpr int NI = WAVE_ROWS / RPI;         // DMA instructions per wave, tile and tensor: 4 or 2
+  constexpr int TILE_BYTES = BN * ROW_BYTES;
+  using M = Mma<DTYPE>;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+  __shared__ __attribute__((aligned(16))) char lds_k0[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char lds_v0[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char lds_k1[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char lds_v1[TILE_BYTES];
+
+  const int per_xcd = gridDim.x >> 3;
+  const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int group = p.H / p.H_kv;
+  if (w >= p.num_tiles * p.H) return;
+  const int hg = w % group;
+  int tile = (w / group) % p.num_tiles;
+  const int kvh = w / (group * p.num_tiles);
+  const int head = kvh * group + hg;
+  int b = 0, q_begin = 0, q_len = 0;
+  for (; b < p.B; ++b) {
+    q_begin = p.cu_q[b];
+    q_len = p.cu_q[b + 1] - q_begin;
+    const int tiles_b = (q_len + BM - 1) / BM;
+    if (tile < tiles_b) break;
+    tile -= tiles_b;
+  }
+  if (b >= p.B) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int li = lane & 15, lg = lane >> 4;
+  const int kv_begin = p.cu_k[b];
+  const int kv_len = p.cu_k[b + 1] - kv_begin;
+  const int q_tile0 = tile * BM;
+  const int q_wave0 = q_tile0 + wave * WQ;
+  int nq_valid = (q_len - q_wave0 + 15) / 16;
+  nq_valid = nq_valid < 0 ? 0 : (nq_valid > NQ16 ? NQ16 : nq_valid);
+  char *out_base = p.out + (int64_t)q_begin * p.o_token_bytes + (int64_t)head * p.o_head_bytes;
+
+  if (kv_len <= 0) {
+    for (int r = tid / CH; r < BM; r += 256 / CH) {
+      const int qr = q_tile0 + r;
+      if (qr < q_len) store16(out_base + (int64_t)qr * p.o_token_bytes + (tid % CH) * 16, vec16{{0, 0, 0, 0}});
+    }
+    return;
+  }
+
+  int shared_len = 0, shift = 0;
+  if (MODE == MODE_QUERY_SIDE) {
+    shared_len = p.shared_kv_lens[b];
+    shared_len = shared_len < 0 ? 0 : (shared_len > kv_len ? kv_len : shared_len);
+    shift = p.affix_shifts[b];
+    if (shift < 0 || shift >= p.rope_rows) shift = 0;
+  }
+
+  vec16 qf[NQ16][KS];
+  vec16 qs[NQ16][KS];
+  const char *q_base = p.q + (int64_t)q_begin * p.q_token_bytes + (int64_t)head * p.q_head_bytes;
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    const int qr = q_wave0 + qt * 16 + li;
+    const bool live = qr < q_len;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[qt][ks] = live ? load16(q_base + (int64_t)qr * p.q_token_bytes + (32 * ks + 8 * lg) * 2)
+                        : vec16{{0, 0, 0, 0}};
+    if (MODE == MODE_QUERY_SIDE) {
+      const float *cr = p.cos_tab + (int64_t)shift * D;
+      const float *sr = p.sin_tab + (int64_t)shift * D;
+#pragma unroll
+      for (int ks = 0; ks < KS / 2; ++ks) {
+        vec16 lo = qf[qt][ks], hi = qf[qt][ks + KS / 2];
+        if (shift != 0) rotate_pair<DTYPE, D>(lo, hi, cr, sr, 32 * ks + 8 * lg, -1.0f);
+        qs[qt][ks] = lo;
+        qs[qt][ks + KS / 2] = hi;
+      }
+    }
+  }
+
+  // ---- DMA bookkeeping: this lane's row and chunk inside each of its NI instructions
+  const int dma_row0 = wave * WAVE_ROWS + lane / CH;   // + i*RPI
+  const int dma_chunk = lane % CH;
+  const char *kc_base = p.k_cache + (int64_t)kvh * p.kv_head_bytes;
+  const char *vc_base = p.v_cache + (int64_t)kvh * p.kv_head_bytes;
+
+  const int tiles_a = (shared_len + BN - 1) / BN;
+  const int tiles_b = (kv_len - shared_len + BN - 1) / BN;
+  const int n_tiles = tiles_a + tiles_b;
+
+  // slots of this lane's rows: even tiles in slot_a, odd tiles in slot_b (two named
+  // register arrays, indexed statically).  load_slots only issues the loads; the
+  // values are first touched by issue() one barrier later, so no wait for them is
+  // ever placed in front of the MFMA work.
+  int slot_a[NI], slot_b[NI];
+  auto load_slots = [&](int t, int (&dst)[NI]) __attribute__((always_inline)) {
+    const TileRange tr = tile_range_of(t < n_tiles ? t : n_tiles - 1, tiles_a, shared_len, kv_len, BN);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int n = tr.n0 + dma_row0 + i * RPI;
+      // rows past the end of the range read index 0 (kv_len > 0, always readable);
+      // issue() ignores the value
+      dst[i] = p.slot_map[kv_begin + ((t < n_tiles && n < tr.n_end) ? n : 0)];
+    }
+  };
+  auto issue = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
+    const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int r = dma_row0 + i * RPI;
+      const uint32_t slot = (uint32_t)slots[i];
+      char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;  // wave-uniform; lane data lands at + lane*16
+      char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
+      // negative slots wrap to huge unsigned values and fail the range test too
+      const bool present = tr.n0 + r < tr.n_end && (uint64_t)slot < (uint64_t)p.num_slots;
+      const int fk = (r / RW) % CH;
+      const int fv = 2 * ((r / RW) % (CH / 2));
+      const char *zero = reinterpret_cast<const char *>(kZeroRow) + (dma_chunk << 4);
+      const uint64_t row_off = (uint64_t)slot * (uint32_t)p.kv_slot_bytes;
+      const char *ksrc = present ? kc_base + row_off + ((dma_chunk ^ fk) << 4) : zero;
+      const char *vsrc = present ? vc_base + row_off + ((dma_chunk ^ fv) << 4) : zero;
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)ksrc,
+                                       (void __attribute__((address_space(3))) *)kdst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)vsrc,
+                                       (void __attribute__((address_space(3))) *)vdst, 16, 0, 0);
+    }
+  };
+
+  float m_run[NQ16], l_run[NQ16];
+  f32x4 o_acc[NQ16][DT];
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    m_run[qt] = -INFINITY;
+    l_run[qt] = 0.0f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = f32x4{0, 0, 0, 0};
+  }
+
+  // lane-constant pieces of the fragment addresses
+  const int k_swz = (li / RW) % CH;                       // f_K of rows 16*nt + li
+  const int v_j = li >> 2, v_ib = li & 3;                 // transpose-read role inside the 16-lane group
+  const int v_row = 4 * lg + v_j;                         // + 32*s (+16 for the second half)
+  const int v_swz = ((v_row / RW) % (CH / 2));            // f_V(row)/2; rows differ by multiples of 16
+  const int v_lane_off = v_row * ROW_BYTES + ((v_ib >> 1) << 4) + ((v_ib & 1) << 3);
+  const float c = p.scale_log2e;
+
+  auto compute = [&](const char *kbuf, const char *vbuf, int n_valid, bool shared_tile) __attribute__((always_inline)) {
+    f32x4 s_acc[NQ16][NT];
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] = f32x4{0, 0, 0, 0};
+    auto scores = [&](const vec16 (&qq)[NQ16][KS]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const vec16 kf = load16(kbuf + (16 * nt + li) * ROW_BYTES + (((4 * ks + lg) ^ k_swz) << 4));
+#pragma unroll
+          for (int qt = 0; qt < NQ16; ++qt)
+            s_acc[qt][nt] = M::run(kf, qq[qt][ks], s_acc[qt][nt]);
+        }
+      }
+    };
+    if (MODE == MODE_QUERY_SIDE && shared_tile) scores(qs);
+    else scores(qf);
+
+    vec16 pf[NQ16][NS];
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) {
+      {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+            mx = fmaxf(mx, s_acc[qt][nt][i]);
+          }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run[qt], mx);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = exp2f((m_run[qt] - m_use) * c);
+        const float mc = m_use * c;
+        float sum = 0.0f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float e = exp2f(s_acc[qt][nt][i] * c - mc);
+            s_acc[qt][nt][i] = e;
+            sum += e;
+          }
+        l_run[qt] = l_run[qt] * alpha + sum;
+        m_run[qt] = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+          pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
+          pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
+          pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
+          pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
+        }
+      }
+    }
+
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int col = (((dt ^ v_swz) & (CH / 2 - 1)) << 5);  // swizzled 32-byte column block of d tile dt
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const char *src = vbuf + v_lane_off + 32 * s * ROW_BYTES + col;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)src);
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4 __attribute__((address_space(3))) *)(src + 16 * ROW_BYTES));
+        vec16 vf;
+        vf.w[0] = (uint32_t)(uint16_t)lo.x | ((uint32_t)(uint16_t)lo.y << 16);
+        vf.w[1] = (uint32_t)(uint16_t)lo.z | ((uint32_t)(uint16_t)lo.w << 16);
+        vf.w[2] = (uint32_t)(uint16_t)hi.x | ((uint32_t)(uint16_t)hi.y << 16);
+        vf.w[3] = (uint32_t)(uint16_t)hi.z | ((uint32_t)(uint16_t)hi.w << 16);
+#pragma unroll
+        for (int qt = 0; qt < NQ16; ++qt)
+          o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
+      }
+    }
+  };
+
+  // ---- two-deep ring: tile t lives in buffer t & 1 ----------------------------------
+  load_slots(0, slot_a);
+  issue(0, lds_k0, lds_v0, slot_a);
+  load_slots(1, slot_b);
+  for (int t = 0; t < n_tiles; t += 2) {
+    int n0, n_end;
+    // even tile: wait for its copies, publish it, start the odd tile, compute
+    __builtin_amdgcn_s_waitcnt(0);  // this wave's copies of tile t have landed
+    __syncthreads();                // ... and everybody else's; buffer 1 is no longer being read
+    if (t + 1 < n_tiles) {
+      load_slots(t + 2, slot_a);    // slot loads go first: vmcnt retires in order, so waiting
+      issue(t + 1, lds_k1, lds_v1, slot_b);  // for them later never waits for the copies behind them
+    }
+    { const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN); n0 = tr.n0; n_end = tr.n_end; }
+    if (nq_valid > 0) compute(lds_k0, lds_v0, n_end - n0, MODE == MODE_QUERY_SIDE && t < tiles_a);
+    if (t + 1 >= n_tiles) break;
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (t + 2 < n_tiles) {
+      load_slots(t + 3, slot_b);
+      issue(t + 2, lds_k0, lds_v0, slot_a);
+    }
+    { const TileRange tr = tile_range_of(t + 1, tiles_a, shared_len, kv_len, BN); n0 = tr.n0; n_end = tr.n_end; }
+    if (nq_valid > 0) compute(lds_k1, lds_v1, n_end - n0, MODE == MODE_QUERY_SIDE && t + 1 < tiles_a);
+  }
+
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
     if (qt < nq_valid) {
@@ -422,13 +748,13 @@ static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStrea
   dim3 grid((unsigned)blocks), block(256);
   switch (mode) {
     case MODE_PLAIN:
-      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_PLAIN>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((varlen_attn_dma_kernel<DTYPE, D, NQ16, MODE_PLAIN>), grid, block, 0, stream, p);
       break;
     case MODE_KEY_SIDE:
       hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_KEY_SIDE>), grid, block, 0, stream, p);
       break;
     default:
-      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_QUERY_SIDE>), grid, block, 0, stream, p);
+      hipLaunchKernelGGL((varlen_attn_dma_kernel<DTYPE, D, NQ16, MODE_QUERY_SIDE>), grid, block, 0, stream, p);
       break;
   }
   return launch_status("varlen_attn_kernel");

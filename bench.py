@@ -85,7 +85,43 @@ def cpu_relocation_baseline(torch, wl, budget_s=20.0):
 
 
 def attention_bench(torch, device, ops, steps, warmup):
-    return None
+    """Anchor-recompute bidirectional varlen attention, one layer call: batch 16, 32 heads (MHA), D = 128, bf16."""
+    from acache_amd.synthetic import attention_batch
+
+    w = attention_batch(seed=0)
+    H = Hkv = 32
+    D, BS = 128, 256
+    gen = torch.Generator(device=device).manual_seed(0)
+    total_q = int(w["cu_q"][-1])
+    q = (torch.randn(total_q, H, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    kc = (torch.randn(w["num_blocks"], BS, Hkv, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    vc = (torch.randn(w["num_blocks"], BS, Hkv, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    cu_q, cu_k, slots = w["cu_q"].to(device), w["cu_k"].to(device), w["slot_map"].to(device)
+
+    def step():
+        return ops.acache_attention(q, kc, vc, cu_q, cu_k, slots)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ms = _event_times_ms(step, steps, torch)
+    avg_ms = sum(ms) / len(ms)
+    flops = 4 * H * D * sum(a * b for a, b in zip(w["q_lens"], w["kv_lens"]))
+    kv_bytes = 2 * sum(w["kv_lens"]) * Hkv * D * 2
+    qo_bytes = 2 * total_q * H * D * 2
+    tflops = flops / (avg_ms * 1e-3) / 1e12
+    return {
+        "metric": "anchor-recompute attn TFLOP/s", "value": round(tflops, 1), "unit": "TFLOP/s",
+        "ms_per_call": round(avg_ms, 4), "min_ms": round(min(ms), 4),
+        "config": {"workload": "configs[3]: batch 16, 32 heads (MHA), D 128, bf16, q = 20% anchors + 32 per request, "
+                               "kv = affix + request + 256 (920-1712), slot map over shared affix slots and shuffled private blocks",
+                   "total_q": total_q, "total_kv": sum(w["kv_lens"])},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "varlen_attn_kernel<bf16,128>", "algorithmic_flops": flops,
+                     "algorithmic_bytes": kv_bytes + qo_bytes,
+                     "achieved_GBps": round((kv_bytes + qo_bytes) / (avg_ms * 1e-3) / 1e9, 1)},
+    }
 
 
 def main():
