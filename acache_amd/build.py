@@ -20,7 +20,7 @@ LIB = PKG / "libacache_hip.so"
 
 # packed-fp32 code generation is switched off for every HIP translation unit
 HIP_FLAGS = [
-    "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    "-O3", "--offload-arch=gfx950", "-std=c++20", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]

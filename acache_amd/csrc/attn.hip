@@ -24,6 +24,9 @@
 namespace acache {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
@@ -65,8 +68,9 @@ template <> struct Mma<ACACHE_BF16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
   }
+  // round-to-nearest-even pair conversion: one v_cvt_pk_bf16_f32 on gfx950
   __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
-    return f32_to_bf16(lo) | (f32_to_bf16(hi) << 16);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
   }
 };
 template <> struct Mma<ACACHE_F16> {
@@ -75,7 +79,7 @@ template <> struct Mma<ACACHE_F16> {
                                                   __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
   }
   __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
-    return f32_to_f16(lo) | (f32_to_f16(hi) << 16);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, f16x2));
   }
 };
 
@@ -349,33 +353,43 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt) {
       {
+        if (n_valid < BN) {  // only the last tile of a range has absent keys
+          asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch, not 64 selects per tile
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
-            mx = fmaxf(mx, s_acc[qt][nt][i]);
-          }
+          for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float m_new = fmaxf(m_run[qt], mx);
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = exp2f((m_run[qt] - m_use) * c);
         const float mc = m_use * c;
+        // rescale the running sum and O only when some query's maximum moved
+        // (wave-uniform test; after the first tiles this is the rare case)
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run[qt]) != 0) {
+          const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * c);
+          l_run[qt] *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+          m_run[qt] = m_new;
+        }
         float sum = 0.0f;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float e = exp2f(s_acc[qt][nt][i] * c - mc);
+            const float e = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
             s_acc[qt][nt][i] = e;
             sum += e;
           }
-        l_run[qt] = l_run[qt] * alpha + sum;
-        m_run[qt] = m_new;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+        l_run[qt] += sum;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
           pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
@@ -631,33 +645,43 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt) {
       {
+        if (n_valid < BN) {  // only the last tile of a range has absent keys
+          asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch, not 64 selects per tile
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
-            mx = fmaxf(mx, s_acc[qt][nt][i]);
-          }
+          for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float m_new = fmaxf(m_run[qt], mx);
         const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = exp2f((m_run[qt] - m_use) * c);
         const float mc = m_use * c;
+        // rescale the running sum and O only when some query's maximum moved
+        // (wave-uniform test; after the first tiles this is the rare case)
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run[qt]) != 0) {
+          const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * c);
+          l_run[qt] *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+          m_run[qt] = m_new;
+        }
         float sum = 0.0f;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float e = exp2f(s_acc[qt][nt][i] * c - mc);
+            const float e = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
             s_acc[qt][nt][i] = e;
             sum += e;
           }
-        l_run[qt] = l_run[qt] * alpha + sum;
-        m_run[qt] = m_new;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+        l_run[qt] += sum;
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
           pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
