@@ -368,18 +368,23 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
           for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run[qt], mx);
-        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float mc = m_use * c;
-        // rescale the running sum and O only when some query's maximum moved
-        // (wave-uniform test; after the first tiles this is the rare case)
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run[qt]) != 0) {
-          const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * c);
+        // m_run is the reference point of the running sum and of O, in log2 units
+        // (score * scale * log2 e).  It only has to stay within 2^8 of the true
+        // running maximum: probabilities up to 256 are harmless in fp32/bf16 and
+        // the final division by the running sum cancels the reference.  So the
+        // rescale of O (64 multiplies per lane) runs only when some query's
+        // maximum jumped by more than 8, which after the first tile is rare.
+        const float mxc = mx * c;
+        if (__builtin_amdgcn_ballot_w64(mxc > m_run[qt] + 8.0f) != 0) {
+          const float m_new = fmaxf(m_run[qt], mxc);
+          const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+          const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
           l_run[qt] *= alpha;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
-          m_run[qt] = m_new;
+          m_run[qt] = m_use;
         }
+        const float mc = m_run[qt];
         float sum = 0.0f;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
@@ -660,18 +665,23 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
           for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run[qt], mx);
-        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float mc = m_use * c;
-        // rescale the running sum and O only when some query's maximum moved
-        // (wave-uniform test; after the first tiles this is the rare case)
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run[qt]) != 0) {
-          const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_use) * c);
+        // m_run is the reference point of the running sum and of O, in log2 units
+        // (score * scale * log2 e).  It only has to stay within 2^8 of the true
+        // running maximum: probabilities up to 256 are harmless in fp32/bf16 and
+        // the final division by the running sum cancels the reference.  So the
+        // rescale of O (64 multiplies per lane) runs only when some query's
+        // maximum jumped by more than 8, which after the first tile is rare.
+        const float mxc = mx * c;
+        if (__builtin_amdgcn_ballot_w64(mxc > m_run[qt] + 8.0f) != 0) {
+          const float m_new = fmaxf(m_run[qt], mxc);
+          const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+          const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
           l_run[qt] *= alpha;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
-          m_run[qt] = m_new;
+          m_run[qt] = m_use;
         }
+        const float mc = m_run[qt];
         float sum = 0.0f;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
