@@ -1,0 +1,167 @@
+"""LLaDA-shaped masked-diffusion transformer for the engine path (torch-ROCm GEMMs + HIP attention).
+
+The reference's nano-vdllm model (nano-vdllm/model/modeling_llada.py) cannot be
+imported without flash-attn and is outside the hot path; the engine only needs a
+model with the same call contract:
+
+    model(input_ids, position_ids=..., logits_keep_indices=None).logits
+    model.model.forward(input_ids=..., position_ids=..., compute_logits=False)
+    model.device
+
+and the same layer shape as LLaDA-8B: pre-norm blocks with RMSNorm, separate
+bias-free q/k/v projections, rotate-half RoPE applied in fp32 at the given
+logical positions (modeling_llada.py:412-453), the paged ``Attention`` module, and
+a SwiGLU MLP; untied output head.  Inputs are ragged ``[T]`` (cache refresh) or
+batched ``[B, L]`` (block refinement), exactly as the runner passes them.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from types import SimpleNamespace
+
+import torch
+from torch import nn
+import torch.nn.functional as F
+
+from .attention import Attention
+from .rope import rope_table
+
+
+@dataclass
+class LLaDAConfig:
+    vocab_size: int = 126464
+    d_model: int = 4096
+    n_heads: int = 32
+    n_kv_heads: int | None = None
+    n_layers: int = 32
+    mlp_hidden_size: int = 12288
+    rope: bool = True
+    rope_theta: float = 500000.0
+    max_sequence_length: int = 4096
+    rms_norm_eps: float = 1e-5
+    mask_token_id: int = 126336
+    weight_tying: bool = False
+
+    @property
+    def effective_n_kv_heads(self) -> int:
+        return self.n_heads if self.n_kv_heads is None else self.n_kv_heads
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.eps = eps
+
+    def forward(self, x):
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
+        return (xf * self.weight.float()).to(x.dtype)
+
+
+class RotaryEmbedding(nn.Module):
+    """fp32 tables ``[max_pos, D]``; ``get_rotary_embedding`` returns ``(sin, cos)`` like the reference (line 372)."""
+
+    def __init__(self, config: LLaDAConfig):
+        super().__init__()
+        self.config = config
+        self.head_dim = config.d_model // config.n_heads
+        self._cos = self._sin = None
+
+    def get_rotary_embedding(self, seq_len: int, device):
+        if self._cos is None or self._cos.shape[0] < seq_len or self._cos.device != torch.device(device):
+            n = max(seq_len, self.config.max_sequence_length)
+            self._cos, self._sin = rope_table(n, self.head_dim, self.config.rope_theta, device=device)
+        return self._sin[:seq_len], self._cos[:seq_len]
+
+    def forward(self, q, k, position_ids, max_pos=None):
+        max_pos = max_pos or self.config.max_sequence_length
+        sin, cos = self.get_rotary_embedding(max_pos, q.device)
+        s = sin[position_ids].unsqueeze(-2)
+        c = cos[position_ids].unsqueeze(-2)
+
+        def rot(x):
+            xf = x.float()
+            h = xf.shape[-1] // 2
+            return (xf * c + torch.cat((-xf[..., h:], xf[..., :h]), -1) * s).type_as(x)
+
+        return rot(q), rot(k)
+
+
+class LLaDABlock(nn.Module):
+    def __init__(self, config: LLaDAConfig):
+        super().__init__()
+        self.config = config
+        d, h, hkv = config.d_model, config.n_heads, config.effective_n_kv_heads
+        self.head_dim = d // h
+        self.attn_norm = RMSNorm(d, config.rms_norm_eps)
+        self.ff_norm = RMSNorm(d, config.rms_norm_eps)
+        self.q_proj = nn.Linear(d, h * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(d, hkv * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(d, hkv * self.head_dim, bias=False)
+        self.attn_out = nn.Linear(h * self.head_dim, d, bias=False)
+        self.ff_proj = nn.Linear(d, config.mlp_hidden_size, bias=False)
+        self.up_proj = nn.Linear(d, config.mlp_hidden_size, bias=False)
+        self.ff_out = nn.Linear(config.mlp_hidden_size, d, bias=False)
+        self.rotary_emb = RotaryEmbedding(config)
+        self.attn = Attention(h, self.head_dim, hkv)
+
+    def forward(self, x, position_ids, max_pos):
+        h, hkv, hd = self.config.n_heads, self.config.effective_n_kv_heads, self.head_dim
+        y = self.attn_norm(x)
+        lead = y.shape[:-1]
+        q = self.q_proj(y).view(*lead, h, hd)
+        k = self.k_proj(y).view(*lead, hkv, hd)
+        v = self.v_proj(y).view(*lead, hkv, hd)
+        if self.config.rope:
+            q, k = self.rotary_emb(q, k, position_ids, max_pos)
+        o = self.attn(q, k, v)
+        x = x + self.attn_out(o.reshape(*lead, h * hd))
+        y = self.ff_norm(x)
+        return x + self.ff_out(F.silu(self.ff_proj(y)) * self.up_proj(y))
+
+
+class LLaDAModel(nn.Module):
+    def __init__(self, config: LLaDAConfig):
+        super().__init__()
+        self.config = config
+        self.transformer = nn.ModuleDict(dict(
+            wte=nn.Embedding(config.vocab_size, config.d_model),
+            blocks=nn.ModuleList([LLaDABlock(config) for _ in range(config.n_layers)]),
+            ln_f=RMSNorm(config.d_model, config.rms_norm_eps),
+            ff_out=nn.Linear(config.d_model, config.vocab_size, bias=False),
+        ))
+
+    def forward(self, input_ids, position_ids=None, compute_logits=True, logits_keep_indices=None):
+        if position_ids is None:
+            position_ids = torch.arange(input_ids.shape[-1], device=input_ids.device).expand_as(input_ids)
+        max_pos = self.config.max_sequence_length
+        x = self.transformer["wte"](input_ids)
+        for block in self.transformer["blocks"]:
+            x = block(x, position_ids, max_pos)
+        if not compute_logits:
+            return SimpleNamespace(logits=None, hidden_states=x)
+        x = self.transformer["ln_f"](x)
+        if logits_keep_indices is not None:  # logits of the listed ragged rows only
+            x = x.reshape(-1, x.shape[-1]).index_select(0, logits_keep_indices)
+        return SimpleNamespace(logits=self.transformer["ff_out"](x))
+
+
+class LLaDAModelLM(nn.Module):
+    """Outer wrapper with the attribute layout the runner walks (``.model.transformer.blocks``)."""
+
+    def __init__(self, config: LLaDAConfig, init_std: float = 0.02):
+        super().__init__()
+        self.config = config
+        self.model = LLaDAModel(config)
+        for p in self.parameters():
+            if p.dim() > 1:
+                nn.init.normal_(p, mean=0.0, std=init_std)
+
+    @property
+    def device(self):
+        return next(self.parameters()).device
+
+    def forward(self, input_ids, position_ids=None, logits_keep_indices=None, compute_logits=True):
+        return self.model(input_ids, position_ids=position_ids, compute_logits=compute_logits,
+                          logits_keep_indices=logits_keep_indices)

@@ -1,0 +1,835 @@
+"""Engine for block-wise masked-diffusion decoding with affix-KV reuse.
+
+Mirror of the reference's ``ModelRunner`` (nano-vdllm/model_runner.py) for the LLaDA
+path: same constructor, attribute names, method names/signatures and return
+values for KV-cache allocation, shared-affix precompute, anchor selection,
+relocation set-up, the ``prepare_*`` context builders and the two generation
+loops.  What is re-designed:
+
+* all device work goes through this package's HIP kernels (scatter, varlen
+  attention, relocation, top-k); anchor top-k for a whole admission batch is one
+  launch of the radix-select kernel instead of ``torch.topk`` + ``sort`` +
+  ``tolist`` per request (model_runner.py:833-843);
+* slot maps, positions and cu_seqlens are assembled with numpy in one pass per
+  call instead of per-token Python loops (model_runner.py:1339-1359);
+* the importance probe observes ``Attention`` through its ``probe`` hook instead
+  of monkey-patching ``forward`` (model_runner.py:730-782);
+* logits are computed only for the rows that are read (``logits_keep_indices``),
+  which the reference does for its Dream path only (model_runner.py:2101-2104);
+* the two generation loops share one implementation.
+
+Not carried over: the dKV-cache schedules (model_runner.py:1725-2030), the Dream
+decoder-layer variants and the CUDA-OOM shrink/retry of the KV cache
+(model_runner.py:592-638) — none is on the affix-KV reuse path measured here.
+"""
+from __future__ import annotations
+
+import math
+import time
+
+import numpy as np
+import torch
+
+from . import ops
+from .block_manager import BlockManager
+from .sequence import Sequence
+from .utils import add_gumbel_noise, get_context, reset_context, set_context
+
+
+class ModelRunner:
+    def __init__(self, model, config):
+        self.config = config
+        self.model = model
+        self.base_model = model.module if hasattr(model, "module") else model
+        self.device = model.device
+        self.kv_cache = None
+        self.kv_cache_block_bytes = 0
+        self.block_manager = None
+        self.shared_prefix_len = 0
+        self.shared_prefix_blocks = 0
+        self.acache_ready = False
+        self.shared_prefix_token_ids: tuple[int, ...] = ()
+        self._affix_relocation_enabled = False
+        self._affix_relocation_max_position = 0
+        self._relocated_affix_slot_offset = None
+        self.profile_timing = bool(getattr(config, "profile_timing", False))
+        self.last_timing = {}
+        self._active_timing = None
+        self.allocate_kv_cache()
+
+    # ------------------------------------------------------------------ model access
+    def _is_dream_model(self):
+        return str(getattr(self.config, "model_type", "")).lower() == "dream"
+
+    def _forward_model(self, input_ids, position_ids=None, compute_logits=True):
+        return self.base_model.model.forward(
+            input_ids=input_ids, position_ids=position_ids, compute_logits=compute_logits)
+
+    def _llada_blocks(self):
+        inner = self.base_model.model
+        if hasattr(inner, "transformer") and "blocks" in inner.transformer:
+            return list(inner.transformer["blocks"])
+        if hasattr(inner, "layers"):
+            return list(inner.layers)
+        raise AttributeError("Unable to locate transformer blocks/layers on model.")
+
+    def _attention_modules(self):
+        return [m for m in self.model.modules() if hasattr(m, "k_cache") and hasattr(m, "v_cache")]
+
+    # ------------------------------------------------------------------ timing (model_runner.py:80-140)
+    def _profile_timing_enabled(self):
+        return self.profile_timing
+
+    def _new_timing(self, mode: str, num_prompts: int):
+        if not self.profile_timing:
+            return None
+        return {"mode": mode, "num_prompts": int(num_prompts)}
+
+    def _start_timing(self):
+        if not self._profile_timing_enabled():
+            return None
+        if self.device.type == "cuda":
+            torch.cuda.synchronize(self.device)
+        return time.perf_counter()
+
+    def _finish_timing(self, timing, key, start):
+        if start is None or timing is None:
+            return
+        if self.device.type == "cuda":
+            torch.cuda.synchronize(self.device)
+        timing[key] = timing.get(key, 0.0) + (time.perf_counter() - start)
+
+    def _add_timing_count(self, timing, key, value=1):
+        if timing is None:
+            return
+        timing[key] = timing.get(key, 0) + int(value)
+
+    def _record_kv_cache_usage(self, timing):
+        if timing is None or self.block_manager is None:
+            return
+        bs = int(self.config.cache_block_size)
+        used = len(self.block_manager.used_block_ids)
+        cap = len(self.block_manager.blocks)
+        timing["kv_cache_block_size"] = bs
+        timing["kv_cache_block_bytes"] = int(self.kv_cache_block_bytes)
+        timing["kv_cache_slot_bytes"] = int(self.kv_cache_block_bytes // bs)
+        for name, value in (("used_blocks", used), ("used_slots", used * bs),
+                            ("used_bytes", used * self.kv_cache_block_bytes),
+                            ("capacity_blocks", cap), ("capacity_slots", cap * bs),
+                            ("capacity_bytes", cap * self.kv_cache_block_bytes)):
+            key = f"kv_cache_peak_{name}"
+            timing[key] = max(timing.get(key, 0), value)
+        timing["kv_cache_peak_used_gb"] = timing["kv_cache_peak_used_bytes"] / 1024 ** 3
+        timing["kv_cache_peak_capacity_gb"] = timing["kv_cache_peak_capacity_bytes"] / 1024 ** 3
+
+    # ------------------------------------------------------------------ KV cache (model_runner.py:142-218)
+    def _reset_acache_state(self):
+        self.shared_prefix_len = 0
+        self.shared_prefix_blocks = 0
+        self.acache_ready = False
+        self.shared_prefix_token_ids = ()
+        self._affix_relocation_enabled = False
+        self._affix_relocation_max_position = 0
+        self._relocated_affix_slot_offset = None
+
+    @staticmethod
+    def _first_attr(obj, *names):
+        for name in names:
+            value = getattr(obj, name, None)
+            if value is not None:
+                return value
+        return None
+
+    def allocate_kv_cache(self, num_blocks: int | None = None):
+        """``kv_cache[2, L, num_blocks, block, H_kv, D]`` bf16 with per-layer views bound to the attention modules."""
+        config, hf = self.config, self.config.hf_config
+        num_heads = self._first_attr(hf, "n_heads", "num_attention_heads")
+        if num_heads is None:
+            raise AttributeError("HF config must define n_heads or num_attention_heads.")
+        num_kv_heads = self._first_attr(hf, "effective_n_kv_heads", "n_kv_heads", "num_key_value_heads") or num_heads
+        hidden = self._first_attr(hf, "d_model", "hidden_size")
+        if hidden is None:
+            raise AttributeError("HF config must define d_model or hidden_size.")
+        num_layers = self._first_attr(hf, "n_layers", "num_hidden_layers")
+        if num_layers is None:
+            raise AttributeError("HF config must define n_layers or num_hidden_layers.")
+        head_dim = hidden // num_heads
+        bs = config.cache_block_size
+        self.kv_cache_block_bytes = 2 * num_layers * bs * num_kv_heads * head_dim * 2  # K and V, bf16
+
+        if num_blocks is None and config.num_kvcache_blocks < 0:
+            free, total = torch.cuda.mem_get_info()
+            stats = torch.cuda.memory_stats()
+            peak, current = stats["allocated_bytes.all.peak"], stats["allocated_bytes.all.current"]
+            reserve = 0
+            if config.enable_acache:
+                reserve = int(max(float(config.acache_memory_reserve_gb), 0.0) * 1024 ** 3)
+            available = total * config.gpu_memory_utilization - (total - free) - peak + current - reserve
+            num_blocks = int(available // self.kv_cache_block_bytes)
+        elif num_blocks is None:
+            num_blocks = config.num_kvcache_blocks
+        config.num_kvcache_blocks = int(num_blocks)
+        assert config.num_kvcache_blocks >= 1, "Not enough GPU memory."
+
+        self.kv_cache = torch.empty(2, num_layers, config.num_kvcache_blocks, bs, num_kv_heads, head_dim,
+                                    dtype=torch.bfloat16, device=self.device)
+        self._reset_acache_state()
+        for layer_id, module in enumerate(self._attention_modules()):
+            module.k_cache = self.kv_cache[0, layer_id]
+            module.v_cache = self.kv_cache[1, layer_id]
+            module.use_reference_attention = self.config.use_reference_attention
+            module.shared_prefix_len = 0
+        self.block_manager = BlockManager(config.num_kvcache_blocks, bs)
+
+    def _shared_affix_k(self, layer_idx: int):
+        h, d = self.kv_cache.shape[-2:]
+        return self.kv_cache[0, layer_idx].view(-1, h, d)[: self.shared_prefix_len]
+
+    # ------------------------------------------------------------------ relocation set-up (231-341)
+    def _configure_affix_relocation(self, seqs: list[Sequence]):
+        uses_rope = bool(getattr(self.config.hf_config, "rope", True))
+        required = uses_rope and any(seq.affix_start != 0 for seq in seqs)
+        max_position = max((len(seq) for seq in seqs), default=0)
+        if not required and not self._affix_relocation_enabled:
+            return
+        if required and self._affix_relocation_enabled and self._affix_relocation_max_position >= max_position:
+            return
+        for block in self._llada_blocks():
+            attention, rotary = block.attn, block.rotary_emb
+            attention.shared_prefix_len = self.shared_prefix_len if required else 0
+            if not required or attention.relocation_rope_cos.shape[0] >= max_position:
+                continue
+            sin, cos = rotary.get_rotary_embedding(max_position, self.device)
+            attention.relocation_rope_cos = cos
+            attention.relocation_rope_sin = sin
+        self._affix_relocation_enabled = required
+        self._affix_relocation_max_position = max_position if required else 0
+
+    def _attention_read_layout(self, seq, use_query_relocation: bool):
+        """Read slots of one request; shared affix slots packed first for query-side relocation (275-282)."""
+        if not use_query_relocation or seq.affix_start == 0:
+            return list(seq.read_slot_map), 0
+        lo = seq.shared_slot_offset
+        hi = lo + self.shared_prefix_len
+        slots = np.asarray(seq.read_slot_map, dtype=np.int64)
+        shared = (slots >= lo) & (slots < hi)
+        return slots[shared].tolist() + slots[~shared].tolist(), int(shared.sum())
+
+    def _use_query_side_affix_relocation(self, relocation_materialized: bool):
+        return (self._affix_relocation_enabled and not relocation_materialized
+                and self.config.max_num_seqs != 1)
+
+    def _reserve_single_sequence_relocation_workspace(self, seq: Sequence, *, force: bool = False):
+        """Pin the blocks right after the shared affix as the destination of its relocated copy (291-312)."""
+        if (self.config.max_num_seqs != 1 and not force) or seq.affix_start == 0:
+            return False
+        bm = self.block_manager
+        if self._relocated_affix_slot_offset is not None:
+            if bm.can_allocate(seq):
+                return True
+            bm.release_prefix_tail(self.shared_prefix_blocks)
+            self._relocated_affix_slot_offset = None
+            return False
+        need = self.shared_prefix_blocks
+        if len(bm.free_block_ids) < need + seq.num_cache_blocks:
+            return False
+        end = self.shared_prefix_blocks + need
+        if any(not bm.blocks[i].is_free for i in range(self.shared_prefix_blocks, end)):
+            return False
+        bm.reserve_prefix(end)
+        self._relocated_affix_slot_offset = self.shared_prefix_blocks * self.config.cache_block_size
+        self._record_kv_cache_usage(self._active_timing)
+        return True
+
+    def _materialize_single_sequence_affix(self, seq: Sequence):
+        """Write the affix copy rotated by ``seq.affix_start`` into the workspace, all layers in one launch (314-341)."""
+        if self._relocated_affix_slot_offset is None or seq.affix_start == 0:
+            seq.relocated_affix_materialized = False
+            return
+        self._configure_affix_relocation([seq])
+        start = self._start_timing()
+        layers = self.kv_cache.shape[1]
+        slots = self.kv_cache.shape[2] * self.kv_cache.shape[3]
+        k_cache = self.kv_cache[0].view(layers, slots, *self.kv_cache.shape[-2:])
+        v_cache = self.kv_cache[1].view_as(k_cache)
+        attention = self._llada_blocks()[0].attn
+        ops.materialize_relocated_affix(
+            k_cache, v_cache, attention.relocation_rope_cos, attention.relocation_rope_sin,
+            self._relocated_affix_slot_offset, seq.affix_len, seq.affix_start)
+        lo, hi = seq.shared_slot_offset, seq.shared_slot_offset + seq.affix_len
+        for local, pos in enumerate(range(seq.affix_start, seq.affix_end)):
+            if lo <= seq.read_slot_map[pos] < hi:
+                seq.read_slot_map[pos] = self._relocated_affix_slot_offset + local
+        seq.relocated_affix_materialized = True
+        self._finish_timing(self._active_timing, "affix_materialize", start)
+
+    # ------------------------------------------------------------------ shared affix (474-541)
+    def _resolve_declared_prefix_tokens(self, seqs: list[Sequence]) -> tuple[int, ...]:
+        if not seqs:
+            return ()
+        affix_len = seqs[0].prompt_affix_len
+        if affix_len <= 0:
+            return ()
+        tokens = tuple(seqs[0].prompt_affix_token_ids)
+        for seq in seqs[1:]:
+            if seq.prompt_affix_len != affix_len:
+                raise ValueError("ACache requires the same explicit affix length for every sequence in the batch.")
+            if tuple(seq.prompt_affix_token_ids) != tokens:
+                raise ValueError("ACache requires identical explicit affix tokens for every sequence in the batch.")
+        return tokens
+
+    def _to_device(self, values, dtype):
+        t = torch.as_tensor(np.asarray(values), dtype=dtype)
+        if self.device.type == "cuda":
+            t = t.pin_memory()
+        return t.to(self.device, non_blocking=True)
+
+    def _precompute_shared_prefix(self, prefix_tokens: list[int]):
+        """One forward of the affix alone at positions ``0..A-1``; its post-RoPE K/V land in slots ``0..A-1``."""
+        n = len(prefix_tokens)
+        if n == 0:
+            return
+        token_ids = tuple(prefix_tokens)
+        if self.acache_ready and self.shared_prefix_token_ids == token_ids:
+            return
+        bs = self.config.cache_block_size
+        shared_blocks = -(-n // bs)
+        self.block_manager.reserve_prefix(shared_blocks)
+        timing = self._active_timing
+        self._record_kv_cache_usage(timing)
+        start = self._start_timing()
+        input_ids = self._to_device(prefix_tokens, torch.int64)
+        positions = torch.arange(n, dtype=torch.int64, device=self.device)
+        cu = self._to_device([0, n], torch.int32)
+        slot_mapping = torch.arange(n, dtype=torch.int32, device=self.device)
+        self._finish_timing(timing, "shared_prefix_prepare", start)
+        set_context(True, cu, cu, None, n, n, slot_mapping, None, total_k=n)
+        modules = self._attention_modules()
+        saved = [m.use_reference_attention for m in modules]
+        try:
+            for m in modules:
+                m.use_reference_attention = True  # attend over the fresh K/V rows, not through block tables
+            start = self._start_timing()
+            self._forward_model(input_ids=input_ids, position_ids=positions, compute_logits=False)
+            self._finish_timing(timing, "shared_prefix_forward", start)
+            self._add_timing_count(timing, "shared_prefix_forward_calls", 1)
+        finally:
+            for m, flag in zip(modules, saved):
+                m.use_reference_attention = flag
+            reset_context()
+        self.shared_prefix_len = n
+        self.shared_prefix_blocks = shared_blocks
+        self.shared_prefix_token_ids = token_ids
+        self.acache_ready = True
+
+    # ------------------------------------------------------------------ anchor selection (543-845)
+    def _compute_anchor_positions(self, seq: Sequence):
+        return self._compute_anchor_positions_batch([seq])[0]
+
+    def _finalize_anchor_selection_probe_layout(self, seq: Sequence, shared_slot_offset: int = 0):
+        """Probe layout: anchor slots reserved but unused; queries = non-affix tokens, affix read from the shared copy."""
+        private = seq.private_slots()
+        dynamic = private[seq.num_anchor_tokens:]
+        assert dynamic.size == seq.num_tokens - seq.affix_len
+        read = np.full(seq.num_tokens, -1, dtype=np.int64)
+        read[seq.affix_start:seq.affix_end] = shared_slot_offset + np.arange(seq.affix_len)
+        outside = seq.non_affix_positions
+        read[outside] = dynamic
+        seq.shared_slot_offset = shared_slot_offset
+        seq.recompute_positions = outside
+        seq.recompute_slot_mapping = dynamic.tolist()
+        seq.read_slot_map = read.tolist()
+
+    def _compute_anchor_positions_batch(self, seqs: list[Sequence]):
+        """Importance of every affix token for each request's [MASK] queries, then per-request top-k.
+
+        Per layer and request: ``softmax(q_mask . K_affix^T * scale)`` over the affix
+        keys only (relocated to the request's ``affix_start``), summed over heads and
+        mask queries into fp32 ``[B, A]`` (model_runner.py:730-773); the K highest
+        (or lowest, ``selection_mode == 'bottom'``) indices, ascending, plus
+        ``affix_start`` are the anchors (833-843; ties go to the lower index).
+        """
+        result = [[] for _ in seqs]
+        active = [(i, s) for i, s in enumerate(seqs) if s.acache_enabled and s.num_anchor_tokens > 0]
+        if not active:
+            return result
+        active_idx = [i for i, _ in active]
+        active_seqs = [s for _, s in active]
+        affix_len = active_seqs[0].affix_len
+        if affix_len <= 0:
+            return result
+        if any(s.affix_len != affix_len for s in active_seqs):
+            raise ValueError("Batched Anchor Selection requires a consistent explicit prefix affix length.")
+
+        timing = self._active_timing
+        start = self._start_timing()
+        importance = torch.zeros(len(active_seqs), affix_len, device=self.device, dtype=torch.float32)
+        saved, temp_allocated, workspace = [], [], False
+        blocks = self._llada_blocks()
+        try:
+            for seq in active_seqs:
+                saved.append((seq, list(seq.block_table), list(seq.anchor_positions), list(seq.recompute_positions),
+                              list(seq.recompute_slot_mapping), list(seq.read_slot_map), seq.shared_slot_offset,
+                              seq.relocated_affix_materialized))
+                if not seq.block_table:
+                    if len(active_seqs) == 1:
+                        workspace = self._reserve_single_sequence_relocation_workspace(seq, force=True)
+                    if not self.block_manager.can_allocate(seq):
+                        raise torch.OutOfMemoryError("Not enough KV cache blocks for anchor-selection probe.")
+                    self.block_manager.allocate(seq)
+                    self._record_kv_cache_usage(timing)
+                    temp_allocated.append(seq)
+                seq.anchor_positions = []
+                self._finalize_anchor_selection_probe_layout(seq)
+                if workspace:
+                    self._materialize_single_sequence_affix(seq)
+
+            input_ids, position_ids, _ = self.prepare_caching_acache(active_seqs, use_query_relocation=False)
+            cu_q = [0]
+            for seq in active_seqs:
+                cu_q.append(cu_q[-1] + len(seq.recompute_positions))
+            mask_rows = input_ids == self.config.mask_id
+            mask_positions = [torch.where(mask_rows[cu_q[b]:cu_q[b + 1]])[0] + cu_q[b] for b in range(len(active_seqs))]
+            self._add_timing_count(timing, "anchor_selection_query_tokens", int(input_ids.numel()))
+            self._add_timing_count(timing, "anchor_selection_kv_tokens", sum(len(s) for s in active_seqs))
+            self._finish_timing(timing, "anchor_selection_prepare", start)
+
+            affix_slots = torch.arange(affix_len, dtype=torch.int32, device=self.device)
+            uses_rope = bool(getattr(self.config.hf_config, "rope", True))
+
+            def make_probe(layer_idx, block):
+                def probe(attention, q):
+                    q_heads = q.reshape(-1, attention.num_heads, attention.head_dim)
+                    rotated = {}
+                    for b, seq in enumerate(active_seqs):
+                        rows = mask_positions[b]
+                        if rows.numel() == 0:
+                            continue
+                        shift = seq.affix_start if uses_rope else 0
+                        if shift not in rotated:
+                            if shift == 0:
+                                rotated[shift] = self._shared_affix_k(layer_idx)
+                            else:  # cached keys sit at positions 0..A-1: move them to affix_start..
+                                sin, cos = block.rotary_emb.get_rotary_embedding(
+                                    max(self._affix_relocation_max_position, shift + 1), self.device)
+                                cache_l = attention.k_cache.view(1, -1, attention.num_kv_heads, attention.head_dim)
+                                deltas = torch.full((affix_len,), shift, dtype=torch.int32, device=self.device)
+                                rotated[shift] = ops.relocate_rope_gather(
+                                    cache_l, attention.v_cache.view_as(cache_l), affix_slots, deltas, cos, sin)[0][0]
+                        affix_k = rotated[shift].permute(1, 0, 2)
+                        groups = attention.num_heads // affix_k.shape[0]
+                        if groups > 1:
+                            affix_k = affix_k.repeat_interleave(groups, dim=0)
+                        seq_q = q_heads.index_select(0, rows).permute(1, 0, 2)
+                        scale = attention.scale if attention.scale is not None else attention.head_dim ** -0.5
+                        weights = torch.softmax(torch.matmul(seq_q, affix_k.transpose(-2, -1)) * scale, dim=-1)
+                        importance[b].add_(weights.sum(dim=-2).sum(dim=-2).float())
+                return probe
+
+            for layer_idx, block in enumerate(blocks):
+                block.attn.probe = make_probe(layer_idx, block)
+            start = self._start_timing()
+            self._forward_model(input_ids=input_ids, position_ids=position_ids, compute_logits=False)
+            self._finish_timing(timing, "anchor_selection_forward", start)
+            self._add_timing_count(timing, "anchor_selection_forward_calls", 1)
+            self._add_timing_count(timing, "anchor_selection_sequences", len(active_seqs))
+        finally:
+            for block in blocks:
+                block.attn.probe = None
+            reset_context()
+            for seq in reversed(temp_allocated):
+                if seq.block_table:
+                    self.block_manager.deallocate(seq)
+            for (seq, table, anchors, rpos, rslots, read, offset, materialized) in saved:
+                seq.block_table = table
+                seq.anchor_positions = anchors
+                seq.recompute_positions = rpos
+                seq.recompute_slot_mapping = rslots
+                seq.read_slot_map = read
+                seq.shared_slot_offset = offset
+                seq.relocated_affix_materialized = materialized
+            if workspace:
+                self.block_manager.release_prefix_tail(self.shared_prefix_blocks)
+                self._relocated_affix_slot_offset = None
+
+        start = self._start_timing()
+        ks = [s.num_anchor_tokens for s in active_seqs]
+        cu_k = np.concatenate([[0], np.cumsum(ks)])
+        cu_a = np.arange(len(active_seqs) + 1) * affix_len
+        chosen = ops.topk_anchors(
+            importance.view(-1), self._to_device(cu_a, torch.int32), self._to_device(cu_k, torch.int32),
+            int(cu_k[-1]), offsets=self._to_device([s.affix_start for s in active_seqs], torch.int32),
+            largest=self.config.selection_mode != "bottom").tolist()
+        for b, i in enumerate(active_idx):
+            result[i] = chosen[cu_k[b]:cu_k[b + 1]]
+        self._finish_timing(timing, "anchor_selection_topk", start)
+        return result
+
+    # ------------------------------------------------------------------ admission (847-1003)
+    def _prepare_acache(self, seqs: list[Sequence]):
+        prefix = self._resolve_declared_prefix_tokens(seqs)
+        if not prefix:
+            return ()
+        for seq in seqs:
+            seq.enable_acache(len(prefix), self.config.anchor_ratio,
+                              affix_start=seq.prompt_affix_start, affix_end=seq.prompt_affix_end)
+        return prefix
+
+    def _select_anchor_positions_for_sequences(self, seqs, prefix_token_ids, allow_kv_cache_resize,
+                                               minimum_blocks=None):
+        # one request per probe forward, as the reference does (model_runner.py:873)
+        for seq in seqs:
+            seq.set_anchor_positions(self._compute_anchor_positions_batch([seq])[0])
+
+    def _prepare_admitted_sequences_for_acache(self, seqs, prefix_token_ids, allow_kv_cache_resize):
+        if not seqs:
+            return
+        if self.acache_ready and self.shared_prefix_token_ids != prefix_token_ids:
+            raise ValueError("ACache prefix mode requires a consistent shared prefix across active requests.")
+        if not self.acache_ready:
+            self._precompute_shared_prefix(list(prefix_token_ids))
+        self._select_anchor_positions_for_sequences(seqs, prefix_token_ids, allow_kv_cache_resize)
+
+    def _finalize_sequence_layout(self, seq: Sequence):
+        seq.finalize_slot_mapping()
+        self._materialize_single_sequence_affix(seq)
+
+    def _collect_admissible_sequences(self, prompts, next_prompt_idx, current_batch_size, max_num_seqs):
+        admissible = []
+        remaining = len(self.block_manager.free_block_ids)
+        while next_prompt_idx < len(prompts) and current_batch_size + len(admissible) < max_num_seqs:
+            seq = prompts[next_prompt_idx]
+            if seq.num_cache_blocks > remaining:
+                break
+            admissible.append(seq)
+            remaining -= seq.num_cache_blocks
+            next_prompt_idx += 1
+        return admissible, next_prompt_idx
+
+    def _admit_sequences_with_acache(self, batched_prompts, new_prompts, prefix_token_ids, allow_kv_cache_resize):
+        if not new_prompts:
+            return 0
+        self._prepare_admitted_sequences_for_acache(new_prompts, prefix_token_ids, allow_kv_cache_resize)
+        self._reserve_single_sequence_relocation_workspace(new_prompts[0])
+        admitted = 0
+        for seq in new_prompts:
+            if not self.block_manager.can_allocate(seq):
+                break
+            self.block_manager.allocate(seq)
+            self._record_kv_cache_usage(self._active_timing)
+            self._finalize_sequence_layout(seq)
+            batched_prompts.append(seq)
+            admitted += 1
+        return admitted
+
+    # ------------------------------------------------------------------ context builders (1004-1114, 1295-1471)
+    def _select(self, seqs, active_indices):
+        if active_indices is None:
+            return list(seqs)
+        if torch.is_tensor(active_indices):
+            active_indices = active_indices.tolist()
+        return [seqs[int(i)] for i in active_indices]
+
+    def prepare_block_tables(self, seqs: list[Sequence]):
+        width = max(len(seq.block_table) for seq in seqs)
+        table = np.full((len(seqs), width), -1, dtype=np.int32)
+        for i, seq in enumerate(seqs):
+            table[i, : len(seq.block_table)] = seq.block_table
+        return self._to_device(table, torch.int32)
+
+    def prepare_caching(self, seqs, active_indices=None):
+        """Full-recompute refresh: every token of every request is a query and is written to its block-table slot."""
+        group = self._select(seqs, active_indices)
+        block_tables = self.prepare_block_tables(group)
+        lens = np.array([len(s) for s in group], dtype=np.int64)
+        cu = np.concatenate([[0], np.cumsum(lens)])
+        input_ids = np.concatenate([np.asarray(s.token_ids, dtype=np.int64) for s in group])
+        positions = np.concatenate([np.arange(n, dtype=np.int64) for n in lens])
+        slot_mapping = np.concatenate([s.private_slots() for s in group])
+        generate_starts = cu[:-1] + np.array([s.generation_start for s in group])
+        current = np.array([s.current_block_idx for s in group])
+        cu_dev = self._to_device(cu, torch.int32)
+        set_context(True, cu_dev, cu_dev, None, int(lens.max()), int(lens.max()),
+                    self._to_device(slot_mapping, torch.int32), block_tables, total_k=int(cu[-1]))
+        return (self._to_device(input_ids, torch.int64), self._to_device(positions, torch.int64),
+                self._to_device(generate_starts, torch.int32), self._to_device(current, torch.int32))
+
+    def prepare_decoding(self, seqs, active_indices=None):
+        """Block refinement on the full-recompute path: the current block's tokens against block-table K/V."""
+        group = self._select(seqs, active_indices)
+        block_length, bs = self.config.block_length, self.config.cache_block_size
+        starts = np.array([s.generation_start + s.current_block_idx * block_length for s in group], dtype=np.int64)
+        seqlens = np.array([len(s) for s in group], dtype=np.int64)
+        positions = starts[:, None] + np.arange(block_length)[None, :]
+        tables = [np.asarray(s.block_table, dtype=np.int64) for s in group]
+        slot_mapping = np.concatenate([t[p // bs] * bs + p % bs for t, p in zip(tables, positions)])
+        block_tables = self.prepare_block_tables(group)
+        set_context(False, None, None, self._to_device(seqlens, torch.int32), None, None,
+                    self._to_device(slot_mapping, torch.int32), block_tables, total_k=int(seqlens.sum()))
+        return self._to_device(positions, torch.int64)
+
+    def _acache_read_side(self, group):
+        relocation_materialized = all(getattr(s, "relocated_affix_materialized", False) for s in group)
+        return relocation_materialized
+
+    def prepare_caching_acache(self, seqs, active_indices=None, use_query_relocation=None):
+        """Cache refresh with affix reuse: queries = anchors + non-affix tokens; keys read through ``read_slot_map``."""
+        group = self._select(seqs, active_indices)
+        self._configure_affix_relocation(group)
+        relocation_materialized = all(getattr(s, "relocated_affix_materialized", False) for s in group)
+        if use_query_relocation is None:
+            use_query_relocation = self.config.max_num_seqs != 1
+        use_query_relocation = (self._affix_relocation_enabled and not relocation_materialized
+                                and bool(use_query_relocation))
+        ids, pos, slots, reads = [], [], [], []
+        shared_lens, shifts, block_starts = [], [], []
+        cu_q, cu_k = [0], [0]
+        for seq in group:
+            q_pos = np.asarray(seq.recompute_positions, dtype=np.int64)
+            assert len(seq.recompute_slot_mapping) == q_pos.size and len(seq.read_slot_map) == len(seq)
+            ids.append(np.asarray(seq.token_ids, dtype=np.int64)[q_pos])
+            pos.append(q_pos)
+            slots.append(np.asarray(seq.recompute_slot_mapping, dtype=np.int64))
+            layout, shared_len = self._attention_read_layout(seq, use_query_relocation)
+            reads.append(np.asarray(layout, dtype=np.int64))
+            shared_lens.append(shared_len)
+            shifts.append(seq.affix_start if self._affix_relocation_enabled else 0)
+            block_starts.append(cu_q[-1] + seq.block_query_start())
+            cu_q.append(cu_q[-1] + q_pos.size)
+            cu_k.append(cu_k[-1] + len(seq))
+        kv_lens = np.diff(cu_k)
+        set_context(
+            True, self._to_device(cu_q, torch.int32), self._to_device(cu_k, torch.int32),
+            self._to_device(kv_lens, torch.int32), int(np.diff(cu_q).max()), int(kv_lens.max()),
+            self._to_device(np.concatenate(slots), torch.int32), None, True,
+            self._to_device(np.concatenate(reads), torch.int32),
+            self._to_device(shared_lens, torch.int32) if use_query_relocation else None,
+            None if relocation_materialized else self._to_device(shifts, torch.int32),
+            total_k=int(cu_k[-1]))
+        return (self._to_device(np.concatenate(ids), torch.int64), self._to_device(np.concatenate(pos), torch.int64),
+                self._to_device(block_starts, torch.int32))
+
+    def prepare_decoding_acache(self, seqs, active_indices=None):
+        """Block refinement with affix reuse: the current block's tokens against the same read slot maps."""
+        group = self._select(seqs, active_indices)
+        block_length = self.config.block_length
+        self._configure_affix_relocation(group)
+        relocation_materialized = all(getattr(s, "relocated_affix_materialized", False) for s in group)
+        use_query_relocation = self._use_query_side_affix_relocation(relocation_materialized)
+        starts, slots, reads, shared_lens, shifts, cu_k = [], [], [], [], [], [0]
+        for seq in group:
+            start = seq.generation_start + seq.current_block_idx * block_length
+            starts.append(start)
+            slots.append(np.asarray(seq.read_slot_map[start:start + block_length], dtype=np.int64))
+            layout, shared_len = self._attention_read_layout(seq, use_query_relocation)
+            reads.append(np.asarray(layout, dtype=np.int64))
+            shared_lens.append(shared_len)
+            shifts.append(seq.affix_start if self._affix_relocation_enabled else 0)
+            cu_k.append(cu_k[-1] + len(seq))
+        kv_lens = np.diff(cu_k)
+        positions = np.asarray(starts, dtype=np.int64)[:, None] + np.arange(block_length)[None, :]
+        cu_q = np.arange(len(group) + 1) * block_length
+        set_context(
+            False, self._to_device(cu_q, torch.int32), self._to_device(cu_k, torch.int32),
+            self._to_device(kv_lens, torch.int32), block_length, int(kv_lens.max()),
+            self._to_device(np.concatenate(slots), torch.int32), None, True,
+            self._to_device(np.concatenate(reads), torch.int32),
+            self._to_device(shared_lens, torch.int32) if use_query_relocation else None,
+            None if relocation_materialized else self._to_device(shifts, torch.int32),
+            total_k=int(cu_k[-1]))
+        return self._to_device(positions, torch.int64)
+
+    # ------------------------------------------------------------------ generation (1473-1723, 2032-2277)
+    @torch.inference_mode()
+    def generate_with_dual_cache(self, prompts: list[Sequence]):
+        """Full affix recompute baseline: every refresh re-encodes the whole request."""
+        return self._generate(prompts, None, "dual_cache")
+
+    @torch.inference_mode()
+    def generate_with_acache(self, prompts: list[Sequence]):
+        """Block-wise denoising with the shared affix K/V reused and only anchors recomputed."""
+        timing = self._new_timing("acache", len(prompts))
+        previous = self._active_timing
+        self._active_timing = timing
+        start = self._start_timing()
+        prefix = self._prepare_acache(prompts)
+        self._finish_timing(timing, "acache_metadata", start)
+        self._active_timing = previous
+        if not prefix:
+            return self.generate_with_dual_cache(prompts)
+        return self._generate(prompts, prefix, "acache", timing)
+
+    def _generate(self, prompts, prefix, mode, timing=None):
+        cfg = self.config
+        device, model = self.device, self.model
+        mask_id, block_length = cfg.mask_id, cfg.block_length
+        temperature, remasking, threshold = cfg.temperature, cfg.remasking, cfg.threshold
+        step = cfg.recompute_batch_size
+        assert step > 0, "recompute_batch_size must be larger than 0"
+        max_num_seqs = cfg.max_num_seqs if cfg.max_num_seqs > 0 else len(prompts)
+        use_acache = prefix is not None
+        if timing is None:
+            timing = self._new_timing(mode, len(prompts))
+        self.last_timing = timing or {}
+        previous = self._active_timing
+        self._active_timing = timing
+        total_start = self._start_timing()
+
+        total_nfe = 0
+        results = [None] * len(prompts)
+        index_of = {seq.seq_id: i for i, seq in enumerate(prompts)}
+        next_idx = 0
+        batch: list[Sequence] = []
+
+        def admit(allow_resize):
+            nonlocal next_idx
+            start = self._start_timing()
+            if use_acache:
+                fresh, next_idx = self._collect_admissible_sequences(prompts, next_idx, len(batch), max_num_seqs)
+                admitted = self._admit_sequences_with_acache(batch, fresh, prefix, allow_resize)
+                next_idx -= len(fresh) - admitted
+            else:
+                while (next_idx < len(prompts) and len(batch) < max_num_seqs
+                       and self.block_manager.can_allocate(prompts[next_idx])):
+                    self.block_manager.allocate(prompts[next_idx])
+                    self._record_kv_cache_usage(timing)
+                    batch.append(prompts[next_idx])
+                    next_idx += 1
+            self._finish_timing(timing, "scheduler", start)
+
+        admit(True)
+        batch_size = len(batch)
+        if batch_size == 0 and prompts:
+            budget = "ACache KV-cache budget" if use_acache else "KV-cache budget"
+            raise RuntimeError(f"No requests could be admitted under the current {budget}.")
+        working = torch.full((batch_size, block_length), mask_id, dtype=torch.int64, device=device)
+        offsets = torch.arange(block_length, device=device)
+
+        def refresh(rows: torch.Tensor):
+            """Cache refresh of the listed batch rows, ``recompute_batch_size`` requests per forward."""
+            nonlocal total_nfe
+            for i in range(0, len(rows), step):
+                part = rows[i:i + step]
+                start = self._start_timing()
+                if use_acache:
+                    input_ids, positions, block_starts = self.prepare_caching_acache(batch, part)
+                    keep = block_starts.unsqueeze(1) + offsets
+                else:
+                    input_ids, positions, gen_starts, current = self.prepare_caching(batch, part)
+                    keep = gen_starts.unsqueeze(1) + block_length * current.unsqueeze(1) + offsets
+                self._finish_timing(timing, "cache_prepare", start)
+                start = self._start_timing()
+                logits = model(input_ids, position_ids=positions, logits_keep_indices=keep.flatten().long()).logits
+                self._finish_timing(timing, "cache_forward", start)
+                self._add_timing_count(timing, "cache_forward_calls", 1)
+                self._add_timing_count(timing, "cache_forward_nfe", len(part))
+                start = self._start_timing()
+                logits = logits.view(len(part), block_length, -1)
+                current_blocks = working[part]
+                x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
+                                                       current_blocks, threshold)
+                r, c = torch.where(transfer)
+                working[part[r], c] = x0[transfer]
+                self._finish_timing(timing, "cache_update", start)
+            total_nfe += len(rows)
+
+        refresh(torch.arange(batch_size, device=device))
+
+        last_active = None
+        refreshed = adjusted = False
+        decoding_positions = None
+        while batch:
+            has_mask = (working == mask_id).any(dim=1)
+            done = ~has_mask
+            if done.any():
+                start = self._start_timing()
+                done_rows = torch.where(done)[0]
+                finished = []
+                for row in done_rows.tolist():
+                    seq = batch[row]
+                    begin = seq.generation_start + seq.current_block_idx * block_length
+                    seq.token_ids[begin:begin + block_length] = working[row].tolist()
+                    seq.current_block_idx += 1
+                    if seq.current_block_idx >= seq.num_blocks_to_generate:
+                        self.block_manager.deallocate(seq)
+                        finished.append(row)
+                        results[index_of[seq.seq_id]] = seq.generated_token_ids
+                working[done_rows] = mask_id
+                if finished:
+                    adjusted = True
+                    gone = set(finished)
+                    batch[:] = [s for i, s in enumerate(batch) if i not in gone]
+                    self._finish_timing(timing, "scheduler", start)
+                    admit(len(batch) == 0)
+                    start = self._start_timing()
+                    survivors = torch.tensor([i for i in range(batch_size) if i not in gone],
+                                             dtype=torch.int64, device=device)
+                    kept = working[survivors]
+                    batch_size = len(batch)
+                    working = torch.full((batch_size, block_length), mask_id, dtype=torch.int64, device=device)
+                    working[: len(survivors)] = kept
+                self._finish_timing(timing, "scheduler", start)
+
+                fresh_rows = torch.where((working == mask_id).all(dim=1))[0]
+                if len(fresh_rows) > 0:
+                    refreshed = True
+                    refresh(fresh_rows)
+                    continue
+
+            if adjusted:
+                adjusted = False
+                has_mask = (working == mask_id).any(dim=1)
+            active = torch.where(has_mask)[0]
+            if len(active) > 0:
+                if last_active is None or len(active) < len(last_active) or refreshed:
+                    refreshed = False
+                    last_active = active
+                    start = self._start_timing()
+                    decoding_positions = (self.prepare_decoding_acache if use_acache else self.prepare_decoding)(
+                        batch, active)
+                    self._finish_timing(timing, "decode_prepare", start)
+                start = self._start_timing()
+                logits = model(working[active], position_ids=decoding_positions).logits
+                self._finish_timing(timing, "decode_forward", start)
+                self._add_timing_count(timing, "decode_forward_calls", 1)
+                self._add_timing_count(timing, "decode_forward_nfe", len(active))
+                start = self._start_timing()
+                current_blocks = working[active]
+                x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
+                                                       current_blocks, threshold)
+                r, c = torch.where(transfer)
+                working[active[r], c] = x0[transfer]
+                self._finish_timing(timing, "decode_update", start)
+                total_nfe += len(active)
+
+        reset_context()
+        self._finish_timing(timing, "total", total_start)
+        if timing is not None:
+            timing["total_nfe"] = int(total_nfe)
+        self._active_timing = previous
+        return results, total_nfe
+
+    # ------------------------------------------------------------------ token transfer (2279-2314)
+    def get_transfer_index(self, logits, temperature, remasking, mask_index, x, threshold=0.9):
+        """Pick the tokens to commit: confidence >= threshold among masked positions, at least one per row."""
+        x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
+        if remasking == "low_confidence":
+            flat = logits.reshape(-1, logits.shape[-1])
+            picks = x0.reshape(-1)
+            conf = torch.empty(picks.shape, dtype=torch.float32, device=logits.device)
+            for lo in range(0, flat.shape[0], 64):  # bounded fp32 temporaries over the vocabulary
+                rows = flat[lo:lo + 64].float()
+                chosen = rows.gather(-1, picks[lo:lo + 64, None]).squeeze(-1)
+                conf[lo:lo + 64] = torch.exp(chosen - torch.logsumexp(rows, dim=-1))
+            x0_p = conf.view_as(x0)
+        elif remasking == "random":
+            x0_p = torch.rand(x0.shape, device=x0.device)
+        else:
+            raise NotImplementedError(remasking)
+        x0 = torch.where(mask_index, x0, x)
+        confidence = torch.where(mask_index, x0_p, torch.full_like(x0_p, -math.inf))
+        transfer = (confidence >= threshold) & mask_index
+        stuck = mask_index.any(dim=1) & ~transfer.any(dim=1)
+        rows = torch.where(stuck)[0]
+        transfer[rows, confidence.argmax(dim=1)[rows]] = True
+        return x0, transfer

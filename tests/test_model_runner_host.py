@@ -1,0 +1,102 @@
+"""ModelRunner host logic that needs no GPU (golden vectors of the reference's CPU tests,
+nano-vdllm/tests/test_model_runner_acache.py:26-61 and 106-124, plus admission failure)."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from acache_amd import Config, Sequence
+from acache_amd.llada import LLaDAConfig, LLaDAModelLM
+from acache_amd.model_runner import ModelRunner
+
+
+def test_attention_read_layout_packs_shared_slots_for_query_relocation():
+    runner = object.__new__(ModelRunner)
+    runner.shared_prefix_len = 3
+    seq = SimpleNamespace(affix_start=2, shared_slot_offset=0, read_slot_map=[8, 9, 0, 10, 2, 11])
+    assert runner._attention_read_layout(seq, True) == ([0, 2, 8, 9, 10, 11], 2)
+
+
+def test_attention_read_layout_keeps_logical_order_for_key_relocation():
+    runner = object.__new__(ModelRunner)
+    runner.shared_prefix_len = 3
+    seq = SimpleNamespace(affix_start=2, shared_slot_offset=0, read_slot_map=[8, 9, 0, 10, 2, 11])
+    assert runner._attention_read_layout(seq, False) == ([8, 9, 0, 10, 2, 11], 0)
+
+
+@pytest.mark.parametrize(
+    ("max_num_seqs", "relocation_materialized", "expected"),
+    [(0, False, True), (16, False, True), (1, False, False), (0, True, False)],
+)
+def test_query_side_relocation_treats_zero_as_unlimited_batching(max_num_seqs, relocation_materialized, expected):
+    runner = object.__new__(ModelRunner)
+    runner._affix_relocation_enabled = True
+    runner.config = SimpleNamespace(max_num_seqs=max_num_seqs)
+    assert runner._use_query_side_affix_relocation(relocation_materialized) is expected
+
+
+def test_profile_timing_helpers_are_noop_when_disabled(monkeypatch):
+    runner = object.__new__(ModelRunner)
+    runner.profile_timing = False
+    runner.device = SimpleNamespace(type="cuda")
+    monkeypatch.setattr(torch.cuda, "synchronize",
+                        lambda *a, **k: pytest.fail("CUDA sync should not run when profile_timing is disabled"))
+    monkeypatch.setattr("acache_amd.model_runner.time.perf_counter",
+                        lambda: pytest.fail("perf_counter should not run when profile_timing is disabled"))
+    assert runner._new_timing("dual_cache", 1) is None
+    assert runner._start_timing() is None
+    runner._finish_timing(None, "total", None)
+    runner._add_timing_count(None, "calls")
+
+
+def _tiny_runner(**overrides):
+    cfg = LLaDAConfig(vocab_size=64, d_model=128, n_heads=2, n_layers=1, mlp_hidden_size=64,
+                      max_sequence_length=64, mask_token_id=63)
+    model = LLaDAModelLM(cfg).to(torch.bfloat16).eval()
+    serve = Config(hf_config=cfg, mask_id=63, recompute_batch_size=2, gen_length=4, block_length=4,
+                   cache_block_size=8, num_kvcache_blocks=2, temperature=0.0, threshold=0.0,
+                   enable_acache=True, anchor_ratio=0.5)
+    for k, v in overrides.items():
+        setattr(serve, k, v)
+    return ModelRunner(model, serve)
+
+
+def test_kv_cache_layout_and_block_bytes_on_cpu():
+    runner = _tiny_runner()
+    assert runner.kv_cache.shape == (2, 1, 2, 8, 2, 64) and runner.kv_cache.dtype == torch.bfloat16
+    assert runner.kv_cache_block_bytes == 2 * 1 * 8 * 2 * 64 * 2
+    attn = runner._llada_blocks()[0].attn
+    assert attn.k_cache.data_ptr() == runner.kv_cache[0, 0].data_ptr()
+    assert attn.v_cache.data_ptr() == runner.kv_cache[1, 0].data_ptr()
+    assert len(runner.block_manager.free_block_ids) == 2
+
+
+def test_block_exhaustion_stops_admission_with_runtime_error():
+    """Failure handling that a host test can force: no request fits the KV budget (model_runner.py:1511-1512, 2080-2081)."""
+    runner = _tiny_runner(num_kvcache_blocks=1)
+    runner.allocate_kv_cache(1)
+    seqs = [Sequence(list(range(2, 14)), gen_length=4, cache_block_size=8, block_length=4, mask_id=63)]  # 16 tokens -> 2 blocks
+    with pytest.raises(RuntimeError, match="No requests could be admitted"):
+        runner.generate_with_dual_cache(seqs)
+
+
+def test_inconsistent_affix_is_rejected_before_any_device_work():
+    runner = _tiny_runner()
+    a = Sequence([2, 3, 4, 5], gen_length=4, cache_block_size=8, block_length=4, mask_id=63, prompt_affix_len=2)
+    b = Sequence([2, 9, 4, 5], gen_length=4, cache_block_size=8, block_length=4, mask_id=63, prompt_affix_len=2)
+    c = Sequence([2, 3, 4, 5], gen_length=4, cache_block_size=8, block_length=4, mask_id=63, prompt_affix_len=3)
+    with pytest.raises(ValueError, match="identical explicit affix tokens"):
+        runner.generate_with_acache([a, b])
+    with pytest.raises(ValueError, match="same explicit affix length"):
+        runner._prepare_acache([a, c])
+    assert runner._prepare_acache([a]) == (2, 3) and a.num_anchor_tokens == 1
+
+
+def test_collect_admissible_sequences_respects_free_blocks():
+    runner = _tiny_runner(num_kvcache_blocks=3)
+    runner.allocate_kv_cache(3)
+    seqs = [Sequence(list(range(2, 14)), gen_length=4, cache_block_size=8, block_length=4, mask_id=63) for _ in range(3)]
+    got, nxt = runner._collect_admissible_sequences(seqs, 0, 0, 8)
+    assert got == seqs[:1] and nxt == 1            # 2 blocks each, 3 free -> one request
+    got, nxt = runner._collect_admissible_sequences(seqs, 0, 0, 0)
+    assert got == [] and nxt == 0
