@@ -124,6 +124,75 @@ def attention_bench(torch, device, ops, steps, warmup):
     }
 
 
+def engine_bench(torch, device, args):
+    """configs[4]: nano-vdllm-style engine step on random-init LLaDA-8B-shaped weights, anchor-ratio sweep
+    against full affix recompute.  Prints one JSON line of its own (not part of the default run)."""
+    import numpy as np
+    from acache_amd import Config, Sequence
+    from acache_amd.llada import LLaDAConfig, LLaDAModelLM
+    from acache_amd.model_runner import ModelRunner
+
+    torch.manual_seed(0)
+    cfg = LLaDAConfig(n_layers=args.engine_layers)
+    with torch.device(device):
+        model = LLaDAModelLM(cfg)
+    model = model.to(torch.bfloat16).eval()
+    # A random output head predicts [MASK] itself once in ~126k tokens; such a position can never be committed
+    # and the decoding loop (the reference's as well) would spin on it.  Trained checkpoints do not do this, so
+    # the synthetic head gets a zero [MASK] row (logit 0, far below the maximum of 126k random logits).
+    with torch.no_grad():
+        model.model.transformer["ff_out"].weight[cfg.mask_token_id].zero_()
+    rng = np.random.default_rng(0)
+    vocab = np.array([t for t in range(cfg.vocab_size) if t != cfg.mask_token_id])
+    affix = rng.choice(vocab, args.engine_affix).tolist()
+    requests = [rng.choice(vocab, int(rng.integers(64, 257))).tolist() for _ in range(args.engine_batch)]
+    gen, block = args.engine_gen, 32
+
+    def prompts():
+        if args.engine_placement == "prefix":
+            return [Sequence(affix + r, gen_length=gen, block_length=block, cache_block_size=256,
+                             mask_id=cfg.mask_token_id, prompt_affix_len=len(affix)) for r in requests]
+        out = []
+        for r in requests:  # infix: request head, affix, request tail
+            cut = len(r) // 2
+            out.append(Sequence(r[:cut] + affix + r[cut:], gen_length=gen, block_length=block, cache_block_size=256,
+                                mask_id=cfg.mask_token_id, prompt_affix_start=cut, prompt_affix_end=cut + len(affix)))
+        return out
+
+    def serve(enable, ratio):
+        return Config(hf_config=cfg, mask_id=cfg.mask_token_id, recompute_batch_size=4, max_num_seqs=0,
+                      gen_length=gen, block_length=block, threshold=0.9, cache_block_size=256,
+                      num_kvcache_blocks=args.engine_kv_blocks, temperature=0.0, enable_acache=enable,
+                      anchor_ratio=ratio, profile_timing=True)
+
+    rows = []
+    for label, enable, ratio in [("full_recompute", False, 0.0)] + [(f"acache_{r}", True, r) for r in args.engine_ratios]:
+        runner = ModelRunner(model, serve(enable, ratio))
+        seqs = prompts()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out, nfe = (runner.generate_with_acache if enable else runner.generate_with_dual_cache)(seqs)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        tokens = sum(len(o) for o in out)
+        timing = {k: round(v, 4) for k, v in runner.last_timing.items() if isinstance(v, float)}
+        rows.append({"mode": label, "anchor_ratio": ratio, "seconds": round(dt, 3), "generated_tokens": tokens,
+                     "tokens_per_s": round(tokens / dt, 1), "nfe": int(nfe), "timing": timing})
+        print(f"[engine] {label}: {tokens / dt:.1f} tok/s, nfe {nfe}, {dt:.2f} s", file=sys.stderr, flush=True)
+        del runner
+        torch.cuda.empty_cache()
+    base = rows[0]["tokens_per_s"]
+    for r in rows:
+        r["speedup_vs_full_recompute"] = round(r["tokens_per_s"] / base, 3)
+    print(json.dumps({
+        "metric": "engine generated tokens/s vs full affix recompute", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"configs[4]: LLaDA-8B shape ({cfg.n_layers} layers, d 4096, 32 heads, vocab 126464), random init, "
+                               f"batch {args.engine_batch}, shared affix {args.engine_affix} ({args.engine_placement}) + 64-256 request tokens, "
+                               f"gen_length {gen}, block_length 32, threshold 0.9 (random weights: ~1 token per step, worst-case NFE)"},
+        "results": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -132,6 +201,14 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="layers of the relocation workload (32 = LLaDA-8B)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-attention", action="store_true")
+    ap.add_argument("--engine", action="store_true", help="run the engine-step sweep (configs[4]) instead")
+    ap.add_argument("--engine-layers", type=int, default=32)
+    ap.add_argument("--engine-batch", type=int, default=16)
+    ap.add_argument("--engine-affix", type=int, default=1000)
+    ap.add_argument("--engine-gen", type=int, default=256)
+    ap.add_argument("--engine-kv-blocks", type=int, default=96)
+    ap.add_argument("--engine-placement", choices=["prefix", "infix"], default="prefix")
+    ap.add_argument("--engine-ratios", type=float, nargs="*", default=[0.0, 0.1, 0.2, 0.3, 0.5, 1.0])
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; --gpus N with N > 1 is not supported "
@@ -146,6 +223,9 @@ def main():
         sys.exit(3)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.engine:
+        engine_bench(torch, device, args)
+        return
 
     wl = build_relocation_workload(torch, device, args.layers)
 
