@@ -343,11 +343,9 @@ class ModelRunner:
     def _compute_anchor_positions_batch(self, seqs: list[Sequence]):
         """Importance of every affix token for each request's [MASK] queries, then per-request top-k.
 
-        Per layer and request: ``softmax(q_mask . K_affix^T * scale)`` over the affix
-        keys only (relocated to the request's ``affix_start``), summed over heads and
-        mask queries into fp32 ``[B, A]`` (model_runner.py:730-773); the K highest
-        (or lowest, ``selection_mode == 'bottom'``) indices, ascending, plus
-        ``affix_start`` are the anchors (833-843; ties go to the lower index).
+        The K highest (or lowest, ``selection_mode == 'bottom'``) importance indices,
+        ascending, plus ``affix_start`` are the anchors (model_runner.py:833-843; ties go
+        to the lower index).  One radix-select launch serves the whole batch.
         """
         result = [[] for _ in seqs]
         active = [(i, s) for i, s in enumerate(seqs) if s.acache_enabled and s.num_anchor_tokens > 0]
@@ -360,7 +358,30 @@ class ModelRunner:
             return result
         if any(s.affix_len != affix_len for s in active_seqs):
             raise ValueError("Batched Anchor Selection requires a consistent explicit prefix affix length.")
+        importance = self._compute_affix_importance(active_seqs)
+        timing = self._active_timing
+        start = self._start_timing()
+        ks = [s.num_anchor_tokens for s in active_seqs]
+        cu_k = np.concatenate([[0], np.cumsum(ks)])
+        cu_a = np.arange(len(active_seqs) + 1) * affix_len
+        chosen = ops.topk_anchors(
+            importance.view(-1), self._to_device(cu_a, torch.int32), self._to_device(cu_k, torch.int32),
+            int(cu_k[-1]), offsets=self._to_device([s.affix_start for s in active_seqs], torch.int32),
+            largest=self.config.selection_mode != "bottom").tolist()
+        for b, i in enumerate(active_idx):
+            result[i] = chosen[cu_k[b]:cu_k[b + 1]]
+        self._finish_timing(timing, "anchor_selection_topk", start)
+        return result
 
+    def _compute_affix_importance(self, active_seqs: list[Sequence]) -> torch.Tensor:
+        """fp32 ``[B, A]`` influence of every shared affix token on each request's [MASK] queries.
+
+        Per layer and request: ``softmax(q_mask . K_affix^T * scale)`` over the affix keys only
+        (the cached keys moved to the request's ``affix_start``), summed over heads and mask
+        queries (model_runner.py:730-773).  Runs one probe forward over the non-affix tokens of
+        the given requests; their layouts and block tables are restored afterwards.
+        """
+        affix_len = active_seqs[0].affix_len
         timing = self._active_timing
         start = self._start_timing()
         importance = torch.zeros(len(active_seqs), affix_len, device=self.device, dtype=torch.float32)
@@ -452,18 +473,7 @@ class ModelRunner:
                 self.block_manager.release_prefix_tail(self.shared_prefix_blocks)
                 self._relocated_affix_slot_offset = None
 
-        start = self._start_timing()
-        ks = [s.num_anchor_tokens for s in active_seqs]
-        cu_k = np.concatenate([[0], np.cumsum(ks)])
-        cu_a = np.arange(len(active_seqs) + 1) * affix_len
-        chosen = ops.topk_anchors(
-            importance.view(-1), self._to_device(cu_a, torch.int32), self._to_device(cu_k, torch.int32),
-            int(cu_k[-1]), offsets=self._to_device([s.affix_start for s in active_seqs], torch.int32),
-            largest=self.config.selection_mode != "bottom").tolist()
-        for b, i in enumerate(active_idx):
-            result[i] = chosen[cu_k[b]:cu_k[b + 1]]
-        self._finish_timing(timing, "anchor_selection_topk", start)
-        return result
+        return importance
 
     # ------------------------------------------------------------------ admission (847-1003)
     def _prepare_acache(self, seqs: list[Sequence]):

@@ -1,0 +1,128 @@
+"""Batch-1 entry points with the HF path's signatures (llada/generate_ACache.py) on the paged engine."""
+import pytest
+import torch
+
+from acache_amd import generate_acache as G
+from acache_amd.llada import LLaDAConfig, LLaDAModelLM
+
+pytestmark = pytest.mark.gpu
+MASK = 63
+
+
+def _model(device, seed=0):
+    torch.manual_seed(seed)
+    cfg = LLaDAConfig(vocab_size=64, d_model=256, n_heads=4, n_layers=2, mlp_hidden_size=128,
+                      max_sequence_length=128, mask_token_id=MASK, rope_theta=10000.0)
+    model = LLaDAModelLM(cfg, init_std=0.08).to(device=device, dtype=torch.bfloat16).eval()
+    with torch.no_grad():
+        model.model.transformer["ff_out"].weight[MASK].zero_()   # a random head must never predict [MASK] itself
+        model.model.transformer["ff_out"].weight[0] += 0.05
+    return cfg, model
+
+
+def test_helpers_match_the_reference_definitions(device):
+    assert [G.ceil_to_int(v) for v in (0.0, 2.0, 2.1, 7.000000000000001)] == [0, 2, 3, 8]
+    x = torch.arange(20, device=device).view(2, 10)
+    anchors = torch.tensor([[1, 3], [0, 2]], device=device)
+    gathered, replace = G.gather_tokens_for_recompute(x, anchors, 6, 8)
+    assert gathered.tolist() == [[1, 3, 6, 7], [10, 12, 16, 17]]
+    assert replace[0].nonzero().flatten().tolist() == [1, 3, 6, 7]
+    mask = torch.tensor([[True] * 7 + [False]], device=device)
+    assert G.get_num_transfer_tokens(mask, 3).tolist() == [[3, 2, 2]]
+    logits = torch.zeros(1, 4, 8, device=device)
+    logits[0, 0, 5] = 9.0
+    logits[0, 2, 1] = 3.0
+    m = torch.tensor([[True, True, True, False]], device=device)
+    cur = torch.full((1, 4), MASK, device=device)
+    x0, t = G.get_transfer_index(logits, 0.0, "low_confidence", m, cur, torch.tensor([2], device=device))
+    assert t.tolist() == [[True, False, True, False]] and x0[0, 0] == 5 and x0[0, 3] == MASK
+    x0, t = G.get_transfer_index(logits, 0.0, "low_confidence", m, cur, None, threshold=0.99)
+    assert t.tolist() == [[True, False, False, False]]
+
+
+@pytest.mark.parametrize("placement", ["prefix", "infix", "suffix"])
+@pytest.mark.parametrize("use_threshold", [True, False])
+def test_generate_with_anchor_attention_fills_the_window(device, placement, use_threshold):
+    cfg, model = _model(device)
+    affix = list(range(20, 36))
+    if placement == "prefix":
+        prompt, kw = affix + [3, 4, 5], dict(affix_start=0, affix_end=16)
+    elif placement == "infix":
+        prompt, kw = [3, 4] + affix + [5, 6], dict(affix_start=2, affix_end=18)
+    else:  # generation window inside the prompt, affix after it
+        prompt, kw = [3, 4] + [MASK] * 8 + affix, dict(affix_start=10, affix_end=26, generation_start=2)
+    x, nfe = G.generate_with_anchor_attention(
+        model, torch.tensor([prompt], device=device), steps=8, gen_length=8, block_length=4, mask_id=MASK,
+        threshold=0.9 if use_threshold else None, anchor_ratio=0.25, **kw)
+    total = len(prompt) + (0 if placement == "suffix" else 8)
+    assert x.shape == (1, total)
+    gen_start = kw.get("generation_start", len(prompt))
+    assert (x[0, gen_start:gen_start + 8] != MASK).all()
+    keep = [i for i in range(len(prompt)) if not gen_start <= i < gen_start + 8]
+    assert x[0, keep].tolist() == [prompt[i] for i in keep]
+    if use_threshold:
+        assert 1 + 2 <= nfe <= 1 + 8
+    else:
+        assert nfe == 1 + 8          # importance pass + exactly `steps` forwards in quota mode
+
+
+def test_precomputed_hf_layout_affix_cache_equals_engine_precompute(device):
+    """A per-layer (k, v) cache in the HF layout ([1, H_kv, A, D], keys before RoPE) lands in the same shared
+    slots as the engine's own affix forward, and generation from it gives the same tokens."""
+    cfg, model = _model(device, seed=2)
+    affix = list(range(10, 40))
+    prompt = [3, 4] + affix + [5, 6, 7]
+    args = dict(steps=8, gen_length=8, block_length=4, mask_id=MASK, threshold=0.9, anchor_ratio=0.2,
+                affix_start=2, affix_end=32)
+    captured = []
+    hooks = []
+    for block in model.model.transformer["blocks"]:
+        store = {}
+        captured.append(store)
+        hooks.append(block.k_proj.register_forward_hook(lambda m, i, o, s=store: s.__setitem__("k", o.detach().clone())))
+        hooks.append(block.v_proj.register_forward_hook(lambda m, i, o, s=store: s.__setitem__("v", o.detach().clone())))
+    runner = G._as_runner(model, mask_id=MASK, block_length=4, gen_length=8, anchor_ratio=0.2, selection_mode="top",
+                          threshold=0.9, temperature=0.0, remasking="low_confidence", total_len=len(prompt) + 8,
+                          affix_len=30)
+    with torch.inference_mode():
+        runner._precompute_shared_prefix(affix)
+    for h in hooks:
+        h.remove()
+    H, D = cfg.n_heads, cfg.d_model // cfg.n_heads
+    hf_cache = tuple((s["k"].view(30, H, D).permute(1, 0, 2).unsqueeze(0), s["v"].view(30, H, D).permute(1, 0, 2).unsqueeze(0))
+                     for s in captured)
+    shared_ref = runner.kv_cache[:, :, 0, :30].clone()
+    x_ref, nfe_ref = G.generate_with_anchor_attention(runner, torch.tensor([prompt], device=device), **args)
+
+    x_hf, nfe_hf = G.generate_with_anchor_attention(model, torch.tensor([prompt], device=device),
+                                                    precomputed_affix_cache=hf_cache, **args)
+    assert torch.equal(x_hf, x_ref) and nfe_hf == nfe_ref
+    runner2 = G._as_runner(model, mask_id=MASK, block_length=4, gen_length=8, anchor_ratio=0.2, selection_mode="top",
+                           threshold=0.9, temperature=0.0, remasking="low_confidence", total_len=len(prompt) + 8,
+                           affix_len=30)
+    G._ingest_affix_cache(runner2, affix, hf_cache)
+    assert torch.equal(runner2.kv_cache[:, :, 0, :30], shared_ref)
+
+
+def test_importance_entry_point_and_anchor_selection(device):
+    cfg, model = _model(device, seed=3)
+    affix = list(range(10, 30))
+    x = torch.tensor([[3, 4] + affix + [5] + [MASK] * 4], device=device)
+    imp = G.compute_attention_importance_cross_affix(model, x, None, mask_id=MASK, affix_start=2, affix_len=20)
+    assert imp.shape == (1, 20) and imp.dtype == torch.float32
+    # softmax rows sum to 1: total importance = mask queries x heads x layers
+    assert abs(imp.sum().item() - 4 * cfg.n_heads * cfg.n_layers) < 0.5
+    idx = G.select_anchor_tokens(imp, 5, "top")
+    assert idx.shape == (1, 5) and idx[0].tolist() == sorted(torch.topk(imp[0], 5).indices.tolist())
+
+
+def test_unsupported_flags_raise(device):
+    cfg, model = _model(device)
+    p = torch.tensor([[3, 4, 5, 6]], device=device)
+    with pytest.raises(NotImplementedError):
+        G.generate_with_anchor_attention(model, p, steps=4, gen_length=4, block_length=4, mask_id=MASK, factor=1.0, affix_end=2)
+    with pytest.raises(NotImplementedError):
+        G.generate_with_anchor_attention(model, p, steps=4, gen_length=4, block_length=4, mask_id=MASK, drop_non_anchor=True, affix_end=2)
+    with pytest.raises(ValueError, match="must not overlap"):
+        G.generate_with_anchor_attention(model, p, steps=2, gen_length=2, block_length=2, mask_id=MASK,
+                                         affix_start=0, affix_end=3, generation_start=2)
