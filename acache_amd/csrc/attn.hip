@@ -108,6 +108,42 @@ __device__ __forceinline__ void rotate_pair(vec16 &lo, vec16 &hi, const float *c
   hi = E::pack(yb);
 }
 
+
+// Which (request, query tile) does global tile index `tile` address?  Lane i loads
+// cu_q[i], cu_q[i+1] for 64 requests at a time, an inclusive wave prefix sum of the
+// per-request tile counts locates the request with one ballot: one memory round
+// trip instead of a dependent scalar load per request.  Returns false when `tile`
+// lies beyond the last live tile.  All lanes return the same values.
+__device__ __forceinline__ bool locate_query_tile(const int32_t *cu_q, int B, int BM, int tile, int &b_out,
+                                                  int &q_begin, int &q_len, int &tile_in_request) {
+  const int lane = threadIdx.x & 63;
+  int base_tiles = 0;
+  for (int b0 = 0; b0 < B; b0 += 64) {
+    const int b = b0 + lane;
+    const int lo = b < B ? cu_q[b] : 0;
+    const int hi = b < B ? cu_q[b + 1] : 0;
+    const int len = hi - lo;
+    const int tiles = b < B && len > 0 ? (len + BM - 1) / BM : 0;
+    int incl = tiles;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (lane >= d) incl += up;
+    }
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(base_tiles + incl > tile);
+    if (hit != 0) {
+      const int src = __builtin_ctzll(hit);
+      b_out = b0 + src;
+      q_begin = __shfl(lo, src);
+      q_len = __shfl(len, src);
+      tile_in_request = tile - base_tiles - (__shfl(incl, src) - __shfl(tiles, src));
+      return true;
+    }
+    base_tiles += __shfl(incl, 63);
+  }
+  return false;
+}
+
 // Key range of tile t: the shared range [0, shared_len) comes first in tiles of BN
 // (query-side mode only, otherwise shared_len = 0), then [shared_len, kv_len).
 struct TileRange {
@@ -152,14 +188,11 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
   const int kvh = w / (group * p.num_tiles);
   const int head = kvh * group + hg;
   int b = 0, q_begin = 0, q_len = 0;
-  for (; b < p.B; ++b) {
-    q_begin = p.cu_q[b];
-    q_len = p.cu_q[b + 1] - q_begin;
-    const int tiles_b = (q_len + BM - 1) / BM;
-    if (tile < tiles_b) break;
-    tile -= tiles_b;
+  {
+    int tile_in_request = 0;
+    if (!locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request)) return;
+    tile = tile_in_request;
   }
-  if (b >= p.B) return;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -499,14 +532,11 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   const int kvh = w / (group * p.num_tiles);
   const int head = kvh * group + hg;
   int b = 0, q_begin = 0, q_len = 0;
-  for (; b < p.B; ++b) {
-    q_begin = p.cu_q[b];
-    q_len = p.cu_q[b + 1] - q_begin;
-    const int tiles_b = (q_len + BM - 1) / BM;
-    if (tile < tiles_b) break;
-    tile -= tiles_b;
+  {
+    int tile_in_request = 0;
+    if (!locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request)) return;
+    tile = tile_in_request;
   }
-  if (b >= p.B) return;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -625,7 +655,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   const int v_lane_off = v_row * ROW_BYTES + ((v_ib >> 1) << 4) + ((v_ib & 1) << 3);
   const float c = p.scale_log2e;
 
-  auto compute = [&](const char *kbuf, const char *vbuf, int n_valid, bool shared_tile) __attribute__((always_inline)) {
+  // MASKED = true: keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
+  auto compute = [&]<bool MASKED>(const char *kbuf, const char *vbuf, int n_valid, bool shared_tile)
+      __attribute__((always_inline)) {
     f32x4 s_acc[NQ16][NT];
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt)
@@ -646,59 +678,65 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     if (MODE == MODE_QUERY_SIDE && shared_tile) scores(qs);
     else scores(qf);
 
+    // Running reference m_run (log2 units: score * scale * log2 e).  It only has to stay within
+    // 2^8 of the true running maximum: probabilities up to 256 are harmless in fp32/bf16 and the
+    // final division by the running sum cancels the reference.  The rescale of O (32 multiplies
+    // per lane and query tile) therefore runs only when some query's maximum jumped by more than
+    // 8 — one wave-uniform test for all query tiles, rarely true after the first key tile.
+    float mxc[NQ16];
+    bool jump = false;
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) {
+      if (MASKED) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      mxc[qt] = mx * c;
+      jump |= mxc[qt] > m_run[qt] + 8.0f;
+    }
+    if (__builtin_amdgcn_ballot_w64(jump) != 0) {
+#pragma unroll
+      for (int qt = 0; qt < NQ16; ++qt) {
+        const float m_new = fmaxf(m_run[qt], mxc[qt]);
+        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
+        l_run[qt] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+        m_run[qt] = m_use;
+      }
+    }
+
     vec16 pf[NQ16][NS];
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt) {
-      {
-        if (n_valid < BN) {  // only the last tile of a range has absent keys
-          asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch, not 64 selects per tile
+      const float mc = m_run[qt];
+      float sum = 0.0f;
 #pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
+      for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+        for (int i = 0; i < 4; ++i) {
+          const float e = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
+          s_acc[qt][nt][i] = e;
+          sum += e;
         }
-        float mx = -INFINITY;
+      l_run[qt] += sum;
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        // m_run is the reference point of the running sum and of O, in log2 units
-        // (score * scale * log2 e).  It only has to stay within 2^8 of the true
-        // running maximum: probabilities up to 256 are harmless in fp32/bf16 and
-        // the final division by the running sum cancels the reference.  So the
-        // rescale of O (64 multiplies per lane) runs only when some query's
-        // maximum jumped by more than 8, which after the first tile is rare.
-        const float mxc = mx * c;
-        if (__builtin_amdgcn_ballot_w64(mxc > m_run[qt] + 8.0f) != 0) {
-          const float m_new = fmaxf(m_run[qt], mxc);
-          const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-          const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
-          l_run[qt] *= alpha;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
-          m_run[qt] = m_use;
-        }
-        const float mc = m_run[qt];
-        float sum = 0.0f;
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float e = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
-            s_acc[qt][nt][i] = e;
-            sum += e;
-          }
-        l_run[qt] += sum;
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-          pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
-          pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
-          pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
-          pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
-        }
+      for (int s = 0; s < NS; ++s) {
+        pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
+        pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
+        pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
+        pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
       }
     }
 
@@ -711,11 +749,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)src);
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (s16x4 __attribute__((address_space(3))) *)(src + 16 * ROW_BYTES));
-        vec16 vf;
-        vf.w[0] = (uint32_t)(uint16_t)lo.x | ((uint32_t)(uint16_t)lo.y << 16);
-        vf.w[1] = (uint32_t)(uint16_t)lo.z | ((uint32_t)(uint16_t)lo.w << 16);
-        vf.w[2] = (uint32_t)(uint16_t)hi.x | ((uint32_t)(uint16_t)hi.y << 16);
-        vf.w[3] = (uint32_t)(uint16_t)hi.z | ((uint32_t)(uint16_t)hi.w << 16);
+        const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+        const vec16 vf{{lo2.x, lo2.y, hi2.x, hi2.y}};  // the two 64-bit results are the operand as is
 #pragma unroll
         for (int qt = 0; qt < NQ16; ++qt)
           o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
@@ -724,11 +759,15 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   };
 
   // ---- two-deep ring: tile t lives in buffer t & 1 ----------------------------------
+  // Full tiles run in the loop without any masking code.  In plain mode the one partial tile (the
+  // tail of the key range) is peeled off behind the loop; with query-side relocation the shared
+  // range may end in a partial tile in the middle, so every tile takes the masked form there.
+  constexpr bool PEEL_TAIL = MODE == MODE_PLAIN;
+  const int n_loop = PEEL_TAIL ? kv_len / BN : n_tiles;  // tiles handled inside the loop
   load_slots(0, slot_a);
   issue(0, lds_k0, lds_v0, slot_a);
   load_slots(1, slot_b);
-  for (int t = 0; t < n_tiles; t += 2) {
-    int n0, n_end;
+  for (int t = 0; t < n_loop; t += 2) {
     // even tile: wait for its copies, publish it, start the odd tile, compute
     __builtin_amdgcn_s_waitcnt(0);  // this wave's copies of tile t have landed
     __syncthreads();                // ... and everybody else's; buffer 1 is no longer being read
@@ -736,36 +775,62 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
       load_slots(t + 2, slot_a);    // slot loads go first: vmcnt retires in order, so waiting
       issue(t + 1, lds_k1, lds_v1, slot_b);  // for them later never waits for the copies behind them
     }
-    { const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN); n0 = tr.n0; n_end = tr.n_end; }
-    if (nq_valid > 0) compute(lds_k0, lds_v0, n_end - n0, MODE == MODE_QUERY_SIDE && t < tiles_a);
-    if (t + 1 >= n_tiles) break;
+    if (nq_valid > 0) {
+      const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
+      compute.template operator()<!PEEL_TAIL>(lds_k0, lds_v0, tr.n_end - tr.n0, MODE == MODE_QUERY_SIDE && t < tiles_a);
+    }
+    if (t + 1 >= n_loop) break;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (t + 2 < n_tiles) {
       load_slots(t + 3, slot_b);
       issue(t + 2, lds_k0, lds_v0, slot_a);
     }
-    { const TileRange tr = tile_range_of(t + 1, tiles_a, shared_len, kv_len, BN); n0 = tr.n0; n_end = tr.n_end; }
-    if (nq_valid > 0) compute(lds_k1, lds_v1, n_end - n0, MODE == MODE_QUERY_SIDE && t + 1 < tiles_a);
+    if (nq_valid > 0) {
+      const TileRange tr = tile_range_of(t + 1, tiles_a, shared_len, kv_len, BN);
+      compute.template operator()<!PEEL_TAIL>(lds_k1, lds_v1, tr.n_end - tr.n0, MODE == MODE_QUERY_SIDE && t + 1 < tiles_a);
+    }
+  }
+  if (PEEL_TAIL && n_loop < n_tiles) {  // tail tile n_loop: its copies were issued one step earlier
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (nq_valid > 0)
+      compute.template operator()<true>((n_loop & 1) ? lds_k1 : lds_k0, (n_loop & 1) ? lds_v1 : lds_v0,
+                                        kv_len - n_loop * BN, false);
   }
 
+  // ---- epilogue: normalise, transpose through LDS, store whole 16-byte chunks ------------------
+  // Lane layout of O^T (query li, features 16*dt + 4*lg .. +4) would give 8-byte stores scattered
+  // over 16 rows; staging the wave's WQ x D tile in LDS (one 16 KiB ring buffer per wave, rows padded
+  // to 272 B against bank conflicts) lets 16 consecutive lanes write one full output row.
+  __syncthreads();  // every wave is done reading the K/V ring
+  {
+    constexpr int OPITCH = ROW_BYTES + 16;
+    static_assert(WQ * OPITCH <= TILE_BYTES, "per-wave output staging must fit one ring buffer");
+    char *stage = wave == 0 ? lds_k0 : wave == 1 ? lds_v0 : wave == 2 ? lds_k1 : lds_v1;
 #pragma unroll
-  for (int qt = 0; qt < NQ16; ++qt) {
-    if (qt < nq_valid) {
+    for (int qt = 0; qt < NQ16; ++qt) {
       float l = l_run[qt];
       l += __shfl_xor(l, 16);
       l += __shfl_xor(l, 32);
       const float inv = l > 0.0f ? 1.0f / l : 1.0f;
-      const int qr = q_wave0 + qt * 16 + li;
-      if (qr < q_len) {
-        char *dst = out_base + (int64_t)qr * p.o_token_bytes + 4 * lg * 2;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-          uint2 val;
-          val.x = M::pack2(o_acc[qt][dt][0] * inv, o_acc[qt][dt][1] * inv);
-          val.y = M::pack2(o_acc[qt][dt][2] * inv, o_acc[qt][dt][3] * inv);
-          *reinterpret_cast<uint2 *>(dst + 16 * dt * 2) = val;
-        }
+      for (int dt = 0; dt < DT; ++dt) {
+        uint2 val;
+        val.x = M::pack2(o_acc[qt][dt][0] * inv, o_acc[qt][dt][1] * inv);
+        val.y = M::pack2(o_acc[qt][dt][2] * inv, o_acc[qt][dt][3] * inv);
+        *reinterpret_cast<uint2 *>(stage + (qt * 16 + li) * OPITCH + (16 * dt + 4 * lg) * 2) = val;
+      }
+    }
+    // same wave wrote and reads: LDS accesses of one wave are ordered, no barrier needed
+    constexpr int ROWS_PER_PASS = 64 / CH;
+#pragma unroll
+    for (int r0 = 0; r0 < WQ; r0 += ROWS_PER_PASS) {
+      const int r = r0 + lane / CH;
+      const int qr = q_wave0 + r;
+      if (qr < q_len) {
+        const vec16 v = load16(stage + r * OPITCH + (lane % CH) * 16);
+        store16(out_base + (int64_t)qr * p.o_token_bytes + (lane % CH) * 16, v);
       }
     }
   }
