@@ -156,6 +156,79 @@ __device__ __forceinline__ TileRange tile_range_of(int t, int tiles_a, int share
   return r;
 }
 
+// Online-softmax update of one key tile, shared by both attention kernels so that they round
+// identically (key-side relocation must reproduce a materialised copy bit for bit).
+//
+// In : s_acc  raw scores S^T of the tile (lane: key rows 16*nt + 4*lg + i, query column li)
+// Out: pf     P^T packed as the B operand of the PV product; m_run / l_acc / o_acc updated.
+//
+// m_run is the reference point of the running sums in log2 units (score * scale * log2 e).  It
+// only has to stay within 2^8 of the true running maximum: probabilities up to 256 are harmless
+// in fp32/bf16 and the final division by the running sum cancels the reference.  The rescale of
+// O (32 multiplies per lane and query tile) therefore runs only when some query's maximum jumped
+// by more than 8 — one wave-uniform test for all query tiles, rarely true after the first tile.
+//
+// l_acc is the running softmax denominator, accumulated by the matrix core as one more row block
+// of O^T whose V^T rows are all ones: every element of l_acc[qt] ends up holding
+// sum_n P[n][query li] of the ROUNDED probabilities, with no VALU adds or cross-lane reduction.
+//
+// MASKED: keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
+template <class M, int NQ16, int NT, int DT, int NS, bool MASKED>
+__device__ __forceinline__ void softmax_tile(f32x4 (&s_acc)[NQ16][NT], float (&m_run)[NQ16],
+                                             f32x4 (&l_acc)[NQ16], f32x4 (&o_acc)[NQ16][DT],
+                                             vec16 (&pf)[NQ16][NS], const vec16 &ones, float c,
+                                             int n_valid, int lg) {
+  float mxc[NQ16];
+  bool jump = false;
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    if (MASKED) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    mxc[qt] = mx * c;
+    jump |= mxc[qt] > m_run[qt] + 8.0f;
+  }
+  if (__builtin_amdgcn_ballot_w64(jump) != 0) {
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) {
+      const float m_new = fmaxf(m_run[qt], mxc[qt]);
+      const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
+      l_acc[qt] *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
+      m_run[qt] = m_use;
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < NQ16; ++qt) {
+    const float mc = m_run[qt];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s_acc[qt][nt][i] = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+      pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
+      pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
+      pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
+      pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
+      l_acc[qt] = M::run(ones, pf[qt][s], l_acc[qt]);
+    }
+  }
+}
+
 template <int DTYPE, int D, int NQ16, int MODE>
 __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
   constexpr int BN = 64;
@@ -327,12 +400,14 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
   };
 
   // ---- running softmax state, one query column per lane -------------------------
-  float m_run[NQ16], l_run[NQ16];
-  f32x4 o_acc[NQ16][DT];
+  float m_run[NQ16];
+  f32x4 o_acc[NQ16][DT], l_acc[NQ16];
+  const uint32_t one2 = M::pack2(1.0f, 1.0f);
+  const vec16 ones{{one2, one2, one2, one2}};
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
     m_run[qt] = -INFINITY;
-    l_run[qt] = 0.0f;
+    l_acc[qt] = f32x4{0, 0, 0, 0};
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = f32x4{0, 0, 0, 0};
   }
@@ -383,60 +458,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
 
     // online softmax; P^T packed straight into the B operand of the PV product
     vec16 pf[NQ16][NS];
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt) {
-      {
-        if (n_valid < BN) {  // only the last tile of a range has absent keys
-          asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch, not 64 selects per tile
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
-        }
-        float mx = -INFINITY;
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        // m_run is the reference point of the running sum and of O, in log2 units
-        // (score * scale * log2 e).  It only has to stay within 2^8 of the true
-        // running maximum: probabilities up to 256 are harmless in fp32/bf16 and
-        // the final division by the running sum cancels the reference.  So the
-        // rescale of O (64 multiplies per lane) runs only when some query's
-        // maximum jumped by more than 8, which after the first tile is rare.
-        const float mxc = mx * c;
-        if (__builtin_amdgcn_ballot_w64(mxc > m_run[qt] + 8.0f) != 0) {
-          const float m_new = fmaxf(m_run[qt], mxc);
-          const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-          const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
-          l_run[qt] *= alpha;
-#pragma unroll
-          for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
-          m_run[qt] = m_use;
-        }
-        const float mc = m_run[qt];
-        float sum = 0.0f;
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float e = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
-            s_acc[qt][nt][i] = e;
-            sum += e;
-          }
-        l_run[qt] += sum;
-#pragma unroll
-        for (int s = 0; s < NS; ++s) {
-          pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
-          pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
-          pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
-          pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
-        }
-      }
-    }
+    softmax_tile<M, NQ16, NT, DT, NS, true>(s_acc, m_run, l_acc, o_acc, pf, ones, c, n_valid, lg);
 
     // O^T += V^T P^T ; lane reads V^T[16*dt + li][keys of slab s, group lg]
 #pragma unroll
@@ -459,9 +481,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
     if (qt < nq_valid) {
-      float l = l_run[qt];
-      l += __shfl_xor(l, 16);
-      l += __shfl_xor(l, 32);
+      const float l = l_acc[qt][0];
       const float inv = l > 0.0f ? 1.0f / l : 1.0f;
       const int qr = q_wave0 + qt * 16 + li;
       if (qr < q_len) {
@@ -614,38 +634,66 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
       dst[i] = p.slot_map[kv_begin + ((t < n_tiles && n < tr.n_end) ? n : 0)];
     }
   };
+  // Per-lane source addresses of row i of a tile, minus the slot term: base + swizzled chunk offset.
+  // One 64-bit multiply-add per row and tensor (slot * row pitch + this) is all the address math
+  // left in the loop.
+  const char *k_lane_src[NI], *v_lane_src[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int r = dma_row0 + i * RPI;
+    k_lane_src[i] = kc_base + ((dma_chunk ^ ((r / RW) % CH)) << 4);
+    v_lane_src[i] = vc_base + ((dma_chunk ^ (2 * ((r / RW) % (CH / 2)))) << 4);
+  }
+  const uint32_t slot_pitch = (uint32_t)p.kv_slot_bytes;
+  const uint32_t slot_limit = p.num_slots > 0x7fffffffLL ? 0x7fffffffu : (uint32_t)p.num_slots;
   auto issue = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
     const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
+    // negative slots wrap to huge unsigned values and fail the range test too
+    bool in_range = true;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int r = dma_row0 + i * RPI;
-      const uint32_t slot = (uint32_t)slots[i];
-      char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;  // wave-uniform; lane data lands at + lane*16
-      char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
-      // negative slots wrap to huge unsigned values and fail the range test too
-      const bool present = tr.n0 + r < tr.n_end && (uint64_t)slot < (uint64_t)p.num_slots;
-      const int fk = (r / RW) % CH;
-      const int fv = 2 * ((r / RW) % (CH / 2));
+    for (int i = 0; i < NI; ++i) in_range &= (uint32_t)slots[i] < slot_limit;
+    const bool all_present = tr.n0 + BN <= tr.n_end && __builtin_amdgcn_ballot_w64(!in_range) == 0;
+    if (all_present) {  // the common case: a full tile whose slots are all inside the cache
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
+        char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;  // wave-uniform; lane data lands at + lane*16
+        char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(k_lane_src[i] + row_off),
+                                         (void __attribute__((address_space(3))) *)kdst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(v_lane_src[i] + row_off),
+                                         (void __attribute__((address_space(3))) *)vdst, 16, 0, 0);
+      }
+    } else {  // last tile of a range, or a slot outside the cache: absent rows come from the zero row
       const char *zero = reinterpret_cast<const char *>(kZeroRow) + (dma_chunk << 4);
-      const uint64_t row_off = (uint64_t)slot * (uint32_t)p.kv_slot_bytes;
-      const char *ksrc = present ? kc_base + row_off + ((dma_chunk ^ fk) << 4) : zero;
-      const char *vsrc = present ? vc_base + row_off + ((dma_chunk ^ fv) << 4) : zero;
-      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)ksrc,
-                                       (void __attribute__((address_space(3))) *)kdst, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)vsrc,
-                                       (void __attribute__((address_space(3))) *)vdst, 16, 0, 0);
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int r = dma_row0 + i * RPI;
+        const bool present = tr.n0 + r < tr.n_end && (uint32_t)slots[i] < slot_limit;
+        const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
+        char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
+        char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
+        const char *ksrc = present ? k_lane_src[i] + row_off : zero;
+        const char *vsrc = present ? v_lane_src[i] + row_off : zero;
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)ksrc,
+                                         (void __attribute__((address_space(3))) *)kdst, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)vsrc,
+                                         (void __attribute__((address_space(3))) *)vdst, 16, 0, 0);
+      }
     }
   };
 
-  float m_run[NQ16], l_run[NQ16];
-  f32x4 o_acc[NQ16][DT];
+  float m_run[NQ16];
+  f32x4 o_acc[NQ16][DT], l_acc[NQ16];
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
     m_run[qt] = -INFINITY;
-    l_run[qt] = 0.0f;
+    l_acc[qt] = f32x4{0, 0, 0, 0};
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = f32x4{0, 0, 0, 0};
   }
+  const uint32_t one2 = M::pack2(1.0f, 1.0f);
+  const vec16 ones{{one2, one2, one2, one2}};
 
   // lane-constant pieces of the fragment addresses
   const int k_swz = (li / RW) % CH;                       // f_K of rows 16*nt + li
@@ -678,67 +726,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     if (MODE == MODE_QUERY_SIDE && shared_tile) scores(qs);
     else scores(qf);
 
-    // Running reference m_run (log2 units: score * scale * log2 e).  It only has to stay within
-    // 2^8 of the true running maximum: probabilities up to 256 are harmless in fp32/bf16 and the
-    // final division by the running sum cancels the reference.  The rescale of O (32 multiplies
-    // per lane and query tile) therefore runs only when some query's maximum jumped by more than
-    // 8 — one wave-uniform test for all query tiles, rarely true after the first key tile.
-    float mxc[NQ16];
-    bool jump = false;
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt) {
-      if (MASKED) {
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
-      }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      mxc[qt] = mx * c;
-      jump |= mxc[qt] > m_run[qt] + 8.0f;
-    }
-    if (__builtin_amdgcn_ballot_w64(jump) != 0) {
-#pragma unroll
-      for (int qt = 0; qt < NQ16; ++qt) {
-        const float m_new = fmaxf(m_run[qt], mxc[qt]);
-        const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
-        l_run[qt] *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
-        m_run[qt] = m_use;
-      }
-    }
-
     vec16 pf[NQ16][NS];
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt) {
-      const float mc = m_run[qt];
-      float sum = 0.0f;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float e = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
-          s_acc[qt][nt][i] = e;
-          sum += e;
-        }
-      l_run[qt] += sum;
-#pragma unroll
-      for (int s = 0; s < NS; ++s) {
-        pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
-        pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
-        pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
-        pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
-      }
-    }
+    softmax_tile<M, NQ16, NT, DT, NS, MASKED>(s_acc, m_run, l_acc, o_acc, pf, ones, c, n_valid, lg);
 
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -810,9 +799,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     char *stage = wave == 0 ? lds_k0 : wave == 1 ? lds_v0 : wave == 2 ? lds_k1 : lds_v1;
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt) {
-      float l = l_run[qt];
-      l += __shfl_xor(l, 16);
-      l += __shfl_xor(l, 32);
+      const float l = l_acc[qt][0];
       const float inv = l > 0.0f ? 1.0f / l : 1.0f;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
