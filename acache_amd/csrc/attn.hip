@@ -156,28 +156,38 @@ __device__ __forceinline__ TileRange tile_range_of(int t, int tiles_a, int share
   return r;
 }
 
-// Online-softmax update of one key tile, shared by both attention kernels so that they round
-// identically (key-side relocation must reproduce a materialised copy bit for bit).
+// Copy 16 bytes per lane from global memory straight into LDS (no register round trip): lane l's
+// bytes land at lds_dst + 16*l, lds_dst being wave-uniform.  The copy is counted by vmcnt; the
+// caller waits (s_waitcnt vmcnt(0)) and synchronises before anybody reads the bytes.
 //
-// In : s_acc  raw scores S^T of the tile (lane: key rows 16*nt + 4*lg + i, query column li)
-// Out: pf     P^T packed as the B operand of the PV product; m_run / l_acc / o_acc updated.
+// Issued from inline assembly rather than __builtin_amdgcn_global_load_lds on purpose: while a
+// copy the compiler knows about is in flight it treats it as a flat access that may touch both
+// memories and turns every later wait for an ordinary LDS read into lgkmcnt(0)/vmcnt(0), which
+// serialises the fragment reads of the matrix loops behind one another.  The leading s_nop covers
+// the wait state the hardware wants between the write of M0 and its use by the copy.
+__device__ __forceinline__ void lds_dma16(const char *src, char *lds_dst) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)lds_dst);
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "{m0}"(base) : "memory");
+}
+
+// Online-softmax update of one key tile, in two steps shared by both attention kernels so that
+// they round identically (key-side relocation must reproduce a materialised copy bit for bit).
 //
-// m_run is the reference point of the running sums in log2 units (score * scale * log2 e).  It
-// only has to stay within 2^8 of the true running maximum: probabilities up to 256 are harmless
-// in fp32/bf16 and the final division by the running sum cancels the reference.  The rescale of
-// O (32 multiplies per lane and query tile) therefore runs only when some query's maximum jumped
-// by more than 8 — one wave-uniform test for all query tiles, rarely true after the first tile.
-//
-// l_acc is the running softmax denominator, accumulated by the matrix core as one more row block
-// of O^T whose V^T rows are all ones: every element of l_acc[qt] ends up holding
-// sum_n P[n][query li] of the ROUNDED probabilities, with no VALU adds or cross-lane reduction.
-//
-// MASKED: keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
-template <class M, int NQ16, int NT, int DT, int NS, bool MASKED>
-__device__ __forceinline__ void softmax_tile(f32x4 (&s_acc)[NQ16][NT], float (&m_run)[NQ16],
-                                             f32x4 (&l_acc)[NQ16], f32x4 (&o_acc)[NQ16][DT],
-                                             vec16 (&pf)[NQ16][NS], const vec16 &ones, float c,
-                                             int n_valid, int lg) {
+// Step 1, softmax_reference: mask absent keys, take the tile's row maxima and move the running
+// reference m_run when needed.
+//   s_acc  raw scores S^T of the tile (lane: key rows 16*nt + 4*lg + i, query column li)
+//   m_run  reference point of the running sums in log2 units (score * scale * log2 e).  It only
+//          has to stay within 2^8 of the true running maximum: probabilities up to 256 are
+//          harmless in fp32/bf16 and the final division by the running sum cancels the reference.
+//          The rescale of O (32 multiplies per lane and query tile) therefore runs only when some
+//          query's maximum jumped by more than 8 — one wave-uniform test for all query tiles,
+//          rarely true after the first tile.
+//   MASKED keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
+template <int NQ16, int NT, int DT, bool MASKED>
+__device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], float (&m_run)[NQ16],
+                                                  f32x4 (&l_acc)[NQ16], f32x4 (&o_acc)[NQ16][DT],
+                                                  float c, int n_valid, int lg) {
   float mxc[NQ16];
   bool jump = false;
 #pragma unroll
@@ -211,21 +221,28 @@ __device__ __forceinline__ void softmax_tile(f32x4 (&s_acc)[NQ16][NT], float (&m
       m_run[qt] = m_use;
     }
   }
+}
+
+// Step 2, softmax_probs_slab: probabilities of the 32-key slab S of the tile, packed as the B
+// operand pf[qt][S] of the PV product, and their contribution to the softmax denominator.
+// l_acc is accumulated by the matrix core as one more row block of O^T whose V^T rows are all
+// ones: every element of l_acc[qt] ends up holding sum_n P[n][query li] of the ROUNDED
+// probabilities, with no VALU adds or cross-lane reduction.  Slabs must be taken in order.
+template <class M, int S, int NQ16, int NT, int NS>
+__device__ __forceinline__ void softmax_probs_slab(const f32x4 (&s_acc)[NQ16][NT], const float (&m_run)[NQ16],
+                                                   f32x4 (&l_acc)[NQ16], vec16 (&pf)[NQ16][NS],
+                                                   const vec16 &ones, float c) {
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
     const float mc = m_run[qt];
+    float e[8];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) s_acc[qt][nt][i] = __builtin_amdgcn_exp2f(s_acc[qt][nt][i] * c - mc);
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      pf[qt][s].w[0] = M::pack2(s_acc[qt][2 * s][0], s_acc[qt][2 * s][1]);
-      pf[qt][s].w[1] = M::pack2(s_acc[qt][2 * s][2], s_acc[qt][2 * s][3]);
-      pf[qt][s].w[2] = M::pack2(s_acc[qt][2 * s + 1][0], s_acc[qt][2 * s + 1][1]);
-      pf[qt][s].w[3] = M::pack2(s_acc[qt][2 * s + 1][2], s_acc[qt][2 * s + 1][3]);
-      l_acc[qt] = M::run(ones, pf[qt][s], l_acc[qt]);
-    }
+    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s_acc[qt][2 * S + (j >> 2)][j & 3] * c - mc);
+    pf[qt][S].w[0] = M::pack2(e[0], e[1]);
+    pf[qt][S].w[1] = M::pack2(e[2], e[3]);
+    pf[qt][S].w[2] = M::pack2(e[4], e[5]);
+    pf[qt][S].w[3] = M::pack2(e[6], e[7]);
+    l_acc[qt] = M::run(ones, pf[qt][S], l_acc[qt]);
   }
 }
 
@@ -458,7 +475,10 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
 
     // online softmax; P^T packed straight into the B operand of the PV product
     vec16 pf[NQ16][NS];
-    softmax_tile<M, NQ16, NT, DT, NS, true>(s_acc, m_run, l_acc, o_acc, pf, ones, c, n_valid, lg);
+    softmax_reference<NQ16, NT, DT, true>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
+    static_assert(NS == 2, "two 32-key slabs per tile");
+    softmax_probs_slab<M, 0>(s_acc, m_run, l_acc, pf, ones, c);
+    softmax_probs_slab<M, 1>(s_acc, m_run, l_acc, pf, ones, c);
 
     // O^T += V^T P^T ; lane reads V^T[16*dt + li][keys of slab s, group lg]
 #pragma unroll
@@ -585,39 +605,40 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     if (shift < 0 || shift >= p.rope_rows) shift = 0;
   }
 
+  const int tiles_a = (shared_len + BN - 1) / BN;
+  const int tiles_b = (kv_len - shared_len + BN - 1) / BN;
+  const int n_tiles = tiles_a + tiles_b;
+
+  // Query fragments (B operand).  Query-side mode scores the shared keys, which come first,
+  // against the rotated query q' and everything after them against q itself; only one of the
+  // two is live at a time: q' is built here and q is re-read when the shared tiles are done.
   vec16 qf[NQ16][KS];
-  vec16 qs[NQ16][KS];
   const char *q_base = p.q + (int64_t)q_begin * p.q_token_bytes + (int64_t)head * p.q_head_bytes;
+  auto load_q = [&](bool rotated) __attribute__((always_inline)) {
 #pragma unroll
-  for (int qt = 0; qt < NQ16; ++qt) {
-    const int qr = q_wave0 + qt * 16 + li;
-    const bool live = qr < q_len;
+    for (int qt = 0; qt < NQ16; ++qt) {
+      const int qr = q_wave0 + qt * 16 + li;
+      const bool live = qr < q_len;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qf[qt][ks] = live ? load16(q_base + (int64_t)qr * p.q_token_bytes + (32 * ks + 8 * lg) * 2)
-                        : vec16{{0, 0, 0, 0}};
-    if (MODE == MODE_QUERY_SIDE) {
-      const float *cr = p.cos_tab + (int64_t)shift * D;
-      const float *sr = p.sin_tab + (int64_t)shift * D;
+      for (int ks = 0; ks < KS; ++ks)
+        qf[qt][ks] = live ? load16(q_base + (int64_t)qr * p.q_token_bytes + (32 * ks + 8 * lg) * 2)
+                          : vec16{{0, 0, 0, 0}};
+      if (MODE == MODE_QUERY_SIDE && rotated && shift != 0) {
+        const float *cr = p.cos_tab + (int64_t)shift * D;
+        const float *sr = p.sin_tab + (int64_t)shift * D;
 #pragma unroll
-      for (int ks = 0; ks < KS / 2; ++ks) {
-        vec16 lo = qf[qt][ks], hi = qf[qt][ks + KS / 2];
-        if (shift != 0) rotate_pair<DTYPE, D>(lo, hi, cr, sr, 32 * ks + 8 * lg, -1.0f);
-        qs[qt][ks] = lo;
-        qs[qt][ks + KS / 2] = hi;
+        for (int ks = 0; ks < KS / 2; ++ks)
+          rotate_pair<DTYPE, D>(qf[qt][ks], qf[qt][ks + KS / 2], cr, sr, 32 * ks + 8 * lg, -1.0f);
       }
     }
-  }
+  };
+  load_q(MODE == MODE_QUERY_SIDE && tiles_a > 0);
 
   // ---- DMA bookkeeping: this lane's row and chunk inside each of its NI instructions
   const int dma_row0 = wave * WAVE_ROWS + lane / CH;   // + i*RPI
   const int dma_chunk = lane % CH;
   const char *kc_base = p.k_cache + (int64_t)kvh * p.kv_head_bytes;
   const char *vc_base = p.v_cache + (int64_t)kvh * p.kv_head_bytes;
-
-  const int tiles_a = (shared_len + BN - 1) / BN;
-  const int tiles_b = (kv_len - shared_len + BN - 1) / BN;
-  const int n_tiles = tiles_a + tiles_b;
 
   // slots of this lane's rows: even tiles in slot_a, odd tiles in slot_b (two named
   // register arrays, indexed statically).  load_slots only issues the loads; the
@@ -659,10 +680,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
         const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
         char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;  // wave-uniform; lane data lands at + lane*16
         char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(k_lane_src[i] + row_off),
-                                         (void __attribute__((address_space(3))) *)kdst, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(v_lane_src[i] + row_off),
-                                         (void __attribute__((address_space(3))) *)vdst, 16, 0, 0);
+        lds_dma16(k_lane_src[i] + row_off, kdst);
+        lds_dma16(v_lane_src[i] + row_off, vdst);
       }
     } else {  // last tile of a range, or a slot outside the cache: absent rows come from the zero row
       const char *zero = reinterpret_cast<const char *>(kZeroRow) + (dma_chunk << 4);
@@ -675,10 +694,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
         char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
         const char *ksrc = present ? k_lane_src[i] + row_off : zero;
         const char *vsrc = present ? v_lane_src[i] + row_off : zero;
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)ksrc,
-                                         (void __attribute__((address_space(3))) *)kdst, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)vsrc,
-                                         (void __attribute__((address_space(3))) *)vdst, 16, 0, 0);
+        lds_dma16(ksrc, kdst);
+        lds_dma16(vsrc, vdst);
       }
     }
   };
@@ -704,7 +721,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   const float c = p.scale_log2e;
 
   // MASKED = true: keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
-  auto compute = [&]<bool MASKED>(const char *kbuf, const char *vbuf, int n_valid, bool shared_tile)
+  auto compute = [&]<bool MASKED>(const char *kbuf, const char *vbuf, int n_valid)
       __attribute__((always_inline)) {
     f32x4 s_acc[NQ16][NT];
 #pragma unroll
@@ -723,17 +740,29 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
         }
       }
     };
-    if (MODE == MODE_QUERY_SIDE && shared_tile) scores(qs);
-    else scores(qf);
+    __builtin_amdgcn_s_setprio(1);
+    scores(qf);
+    // Issue order of this region: K fragments are read four fragments (eight matrix
+    // instructions) ahead of their use, so LDS latency hides behind the matrix core.
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < (NT * KS - 4) / 2; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 * NQ16, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4 * NQ16, 0);
+    __builtin_amdgcn_s_setprio(0);
 
+    softmax_reference<NQ16, NT, DT, MASKED>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
+
+    // O^T += V^T P^T, one 32-key slab at a time, so that the exponentials of the second slab
+    // have the matrix-core work of the first to hide behind.
+    static_assert(NS == 2, "two 32-key slabs per tile");
     vec16 pf[NQ16][NS];
-    softmax_tile<M, NQ16, NT, DT, NS, MASKED>(s_acc, m_run, l_acc, o_acc, pf, ones, c, n_valid, lg);
-
+    auto pv_slab = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const int col = (((dt ^ v_swz) & (CH / 2 - 1)) << 5);  // swizzled 32-byte column block of d tile dt
-#pragma unroll
-      for (int s = 0; s < NS; ++s) {
+      for (int dt = 0; dt < DT; ++dt) {
+        const int col = (((dt ^ v_swz) & (CH / 2 - 1)) << 5);  // swizzled 32-byte column block of d tile dt
         const char *src = vbuf + v_lane_off + 32 * s * ROW_BYTES + col;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)src);
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
@@ -744,7 +773,21 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
         for (int qt = 0; qt < NQ16; ++qt)
           o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
       }
+    };
+    softmax_probs_slab<M, 0>(s_acc, m_run, l_acc, pf, ones, c);
+    __builtin_amdgcn_s_setprio(1);
+    pv_slab(0);
+    softmax_probs_slab<M, 1>(s_acc, m_run, l_acc, pf, ones, c);
+    pv_slab(1);
+    // Issue order: V fragments two d-tiles ahead of their use.
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < 2 * DT - 2; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, NQ16, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x008, 3 * NQ16, 0);
+    __builtin_amdgcn_s_setprio(0);
   };
 
   // ---- two-deep ring: tile t lives in buffer t & 1 ----------------------------------
@@ -765,8 +808,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
       issue(t + 1, lds_k1, lds_v1, slot_b);  // for them later never waits for the copies behind them
     }
     if (nq_valid > 0) {
+      if (MODE == MODE_QUERY_SIDE && t == tiles_a && t > 0) load_q(false);  // shared keys done: back to q
       const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
-      compute.template operator()<!PEEL_TAIL>(lds_k0, lds_v0, tr.n_end - tr.n0, MODE == MODE_QUERY_SIDE && t < tiles_a);
+      compute.template operator()<!PEEL_TAIL>(lds_k0, lds_v0, tr.n_end - tr.n0);
     }
     if (t + 1 >= n_loop) break;
     __builtin_amdgcn_s_waitcnt(0);
@@ -776,8 +820,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
       issue(t + 2, lds_k0, lds_v0, slot_a);
     }
     if (nq_valid > 0) {
+      if (MODE == MODE_QUERY_SIDE && t + 1 == tiles_a) load_q(false);
       const TileRange tr = tile_range_of(t + 1, tiles_a, shared_len, kv_len, BN);
-      compute.template operator()<!PEEL_TAIL>(lds_k1, lds_v1, tr.n_end - tr.n0, MODE == MODE_QUERY_SIDE && t + 1 < tiles_a);
+      compute.template operator()<!PEEL_TAIL>(lds_k1, lds_v1, tr.n_end - tr.n0);
     }
   }
   if (PEEL_TAIL && n_loop < n_tiles) {  // tail tile n_loop: its copies were issued one step earlier
@@ -785,7 +830,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     __syncthreads();
     if (nq_valid > 0)
       compute.template operator()<true>((n_loop & 1) ? lds_k1 : lds_k0, (n_loop & 1) ? lds_v1 : lds_v0,
-                                        kv_len - n_loop * BN, false);
+                                        kv_len - n_loop * BN);
   }
 
   // ---- epilogue: normalise, transpose through LDS, store whole 16-byte chunks ------------------
