@@ -667,36 +667,47 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   }
   const uint32_t slot_pitch = (uint32_t)p.kv_slot_bytes;
   const uint32_t slot_limit = p.num_slots > 0x7fffffffLL ? 0x7fffffffu : (uint32_t)p.num_slots;
-  auto issue = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
+  // A tile whose 64 rows all exist and whose slots all lie inside the cache (the common case) is
+  // copied row group by row group with issue_rows(), which the compute phase spreads over its
+  // own instruction stream: four waves issuing all their copies at once right behind the barrier
+  // queue up in the vector memory path for about a thousand cycles, during which they cannot
+  // issue anything else.  Every other tile takes issue_slow(): absent rows come from the zero row.
+  auto all_present = [&](int t, const int (&slots)[NI]) __attribute__((always_inline)) {
     const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
-    // negative slots wrap to huge unsigned values and fail the range test too
-    bool in_range = true;
+    bool in_range = true;  // negative slots wrap to huge unsigned values and fail the range test too
 #pragma unroll
     for (int i = 0; i < NI; ++i) in_range &= (uint32_t)slots[i] < slot_limit;
-    const bool all_present = tr.n0 + BN <= tr.n_end && __builtin_amdgcn_ballot_w64(!in_range) == 0;
-    if (all_present) {  // the common case: a full tile whose slots are all inside the cache
+    return tr.n0 + BN <= tr.n_end && __builtin_amdgcn_ballot_w64(!in_range) == 0;
+  };
+  auto issue_rows = [&](int i, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
+    const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
+    char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;  // wave-uniform; lane data lands at + lane*16
+    char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
+    lds_dma16(k_lane_src[i] + row_off, kdst);
+    lds_dma16(v_lane_src[i] + row_off, vdst);
+  };
+  auto issue_slow = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
+    const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
+    const char *zero = reinterpret_cast<const char *>(kZeroRow) + (dma_chunk << 4);
 #pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
-        char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;  // wave-uniform; lane data lands at + lane*16
-        char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
-        lds_dma16(k_lane_src[i] + row_off, kdst);
-        lds_dma16(v_lane_src[i] + row_off, vdst);
-      }
-    } else {  // last tile of a range, or a slot outside the cache: absent rows come from the zero row
-      const char *zero = reinterpret_cast<const char *>(kZeroRow) + (dma_chunk << 4);
+    for (int i = 0; i < NI; ++i) {
+      const int r = dma_row0 + i * RPI;
+      const bool present = tr.n0 + r < tr.n_end && (uint32_t)slots[i] < slot_limit;
+      const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
+      char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
+      char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
+      const char *ksrc = present ? k_lane_src[i] + row_off : zero;
+      const char *vsrc = present ? v_lane_src[i] + row_off : zero;
+      lds_dma16(ksrc, kdst);
+      lds_dma16(vsrc, vdst);
+    }
+  };
+  auto issue = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
+    if (all_present(t, slots)) {
 #pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int r = dma_row0 + i * RPI;
-        const bool present = tr.n0 + r < tr.n_end && (uint32_t)slots[i] < slot_limit;
-        const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
-        char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
-        char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
-        const char *ksrc = present ? k_lane_src[i] + row_off : zero;
-        const char *vsrc = present ? v_lane_src[i] + row_off : zero;
-        lds_dma16(ksrc, kdst);
-        lds_dma16(vsrc, vdst);
-      }
+      for (int i = 0; i < NI; ++i) issue_rows(i, kbuf, vbuf, slots);
+    } else {
+      issue_slow(t, kbuf, vbuf, slots);
     }
   };
 
@@ -721,8 +732,17 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   const float c = p.scale_log2e;
 
   // MASKED = true: keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
-  auto compute = [&]<bool MASKED>(const char *kbuf, const char *vbuf, int n_valid)
-      __attribute__((always_inline)) {
+  // stepped: the copies of the next tile (into nk / nv, slots nslots) ride along, one row group at
+  // each of four points of this tile's work.
+  auto compute = [&]<bool MASKED>(const char *kbuf, const char *vbuf, int n_valid, bool stepped, char *nk,
+                                  char *nv, const int (&nslots)[NI]) __attribute__((always_inline)) {
+    auto copy_point = [&](int point) __attribute__((always_inline)) {
+      if (stepped) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+          if (i * 4 / NI == point) issue_rows(i, nk, nv, nslots);
+      }
+    };
     f32x4 s_acc[NQ16][NT];
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt)
@@ -740,6 +760,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
         }
       }
     };
+    copy_point(0);
     __builtin_amdgcn_s_setprio(1);
     scores(qf);
     // Issue order of this region: K fragments are read four fragments (eight matrix
@@ -753,7 +774,9 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     __builtin_amdgcn_sched_group_barrier(0x008, 4 * NQ16, 0);
     __builtin_amdgcn_s_setprio(0);
 
+    copy_point(1);
     softmax_reference<NQ16, NT, DT, MASKED>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
+    copy_point(2);
 
     // O^T += V^T P^T, one 32-key slab at a time, so that the exponentials of the second slab
     // have the matrix-core work of the first to hide behind.
@@ -775,6 +798,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
       }
     };
     softmax_probs_slab<M, 0>(s_acc, m_run, l_acc, pf, ones, c);
+    copy_point(3);
     __builtin_amdgcn_s_setprio(1);
     pv_slab(0);
     softmax_probs_slab<M, 1>(s_acc, m_run, l_acc, pf, ones, c);
@@ -803,26 +827,36 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     // even tile: wait for its copies, publish it, start the odd tile, compute
     __builtin_amdgcn_s_waitcnt(0);  // this wave's copies of tile t have landed
     __syncthreads();                // ... and everybody else's; buffer 1 is no longer being read
+    bool stepped = false;
     if (t + 1 < n_tiles) {
       load_slots(t + 2, slot_a);    // slot loads go first: vmcnt retires in order, so waiting
-      issue(t + 1, lds_k1, lds_v1, slot_b);  // for them later never waits for the copies behind them
+      stepped = all_present(t + 1, slot_b);  // for them later never waits for the copies behind them
+      if (!stepped) issue_slow(t + 1, lds_k1, lds_v1, slot_b);
     }
     if (nq_valid > 0) {
       if (MODE == MODE_QUERY_SIDE && t == tiles_a && t > 0) load_q(false);  // shared keys done: back to q
       const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
-      compute.template operator()<!PEEL_TAIL>(lds_k0, lds_v0, tr.n_end - tr.n0);
+      compute.template operator()<!PEEL_TAIL>(lds_k0, lds_v0, tr.n_end - tr.n0, stepped, lds_k1, lds_v1, slot_b);
+    } else if (stepped) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) issue_rows(i, lds_k1, lds_v1, slot_b);
     }
     if (t + 1 >= n_loop) break;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    stepped = false;
     if (t + 2 < n_tiles) {
       load_slots(t + 3, slot_b);
-      issue(t + 2, lds_k0, lds_v0, slot_a);
+      stepped = all_present(t + 2, slot_a);
+      if (!stepped) issue_slow(t + 2, lds_k0, lds_v0, slot_a);
     }
     if (nq_valid > 0) {
       if (MODE == MODE_QUERY_SIDE && t + 1 == tiles_a) load_q(false);
       const TileRange tr = tile_range_of(t + 1, tiles_a, shared_len, kv_len, BN);
-      compute.template operator()<!PEEL_TAIL>(lds_k1, lds_v1, tr.n_end - tr.n0);
+      compute.template operator()<!PEEL_TAIL>(lds_k1, lds_v1, tr.n_end - tr.n0, stepped, lds_k0, lds_v0, slot_a);
+    } else if (stepped) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) issue_rows(i, lds_k0, lds_v0, slot_a);
     }
   }
   if (PEEL_TAIL && n_loop < n_tiles) {  // tail tile n_loop: its copies were issued one step earlier
@@ -830,7 +864,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     __syncthreads();
     if (nq_valid > 0)
       compute.template operator()<true>((n_loop & 1) ? lds_k1 : lds_k0, (n_loop & 1) ? lds_v1 : lds_v0,
-                                        kv_len - n_loop * BN);
+                                        kv_len - n_loop * BN, false, nullptr, nullptr, slot_a);
   }
 
   // ---- epilogue: normalise, transpose through LDS, store whole 16-byte chunks ------------------
