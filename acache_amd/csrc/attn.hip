@@ -146,6 +146,34 @@ __device__ __forceinline__ bool locate_query_tile(const int32_t *cu_q, int B, in
 
 // Key range of tile t: the shared range [0, shared_len) comes first in tiles of BN
 // (query-side mode only, otherwise shared_len = 0), then [shared_len, kv_len).
+// Same lookup, but over the requests sorted by descending key count (ties: lower index first), for
+// batches of up to 64 requests.  A block's run time is proportional to its request's key count
+// and the hardware hands out blocks in index order, so this is longest-processing-time-first
+// list scheduling: the short blocks fill the gaps at the end instead of the long ones sticking out.
+__device__ __forceinline__ bool locate_query_tile_lpt(const int32_t *cu_q, const int32_t *cu_k, int B, int BM,
+                                                      int rank, int &b_out, int &q_begin, int &q_len,
+                                                      int &tile_in_request) {
+  const int lane = threadIdx.x & 63;
+  const int lo = lane < B ? cu_q[lane] : 0;
+  const int len = lane < B ? cu_q[lane + 1] - lo : 0;
+  const int kv = lane < B ? cu_k[lane + 1] - cu_k[lane] : 0;
+  const int tiles = len > 0 ? (len + BM - 1) / BM : 0;
+  int before = 0;  // query tiles of the requests sorted in front of this lane's request
+  for (int j = 0; j < B; ++j) {
+    const int kv_j = __builtin_amdgcn_readlane(kv, j);
+    const int tiles_j = __builtin_amdgcn_readlane(tiles, j);
+    if (kv_j > kv || (kv_j == kv && j < lane)) before += tiles_j;
+  }
+  const uint64_t hit = __builtin_amdgcn_ballot_w64(lane < B && rank >= before && rank < before + tiles);
+  if (hit == 0) return false;
+  const int src = __builtin_ctzll(hit);
+  b_out = src;
+  q_begin = __shfl(lo, src);
+  q_len = __shfl(len, src);
+  tile_in_request = rank - __shfl(before, src);
+  return true;
+}
+
 struct TileRange {
   int n0, n_end;
 };
@@ -563,18 +591,36 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   __shared__ __attribute__((aligned(16))) char lds_k1[TILE_BYTES];
   __shared__ __attribute__((aligned(16))) char lds_v1[TILE_BYTES];
 
+  // Block -> (query tile, head).  Consecutive block indices go to different XCDs (index mod 8), each
+  // with its own L2, so every XCD is given a contiguous range of KV heads: all query tiles that
+  // read a head's K/V find it in the same L2.  When the KV heads divide evenly among the XCDs,
+  // an XCD walks the query tiles in the outer loop (longest request first, see
+  // locate_query_tile_lpt) and its heads in the inner one; otherwise heads are outermost.
   const int per_xcd = gridDim.x >> 3;
-  const int w = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
   const int group = p.H / p.H_kv;
-  if (w >= p.num_tiles * p.H) return;
-  const int hg = w % group;
-  int tile = (w / group) % p.num_tiles;
-  const int kvh = w / (group * p.num_tiles);
+  int tile, kvh, hg;
+  if (p.H_kv % 8 == 0) {
+    const int heads_per_xcd = (p.H_kv >> 3) * group;
+    tile = idx / heads_per_xcd;
+    if (tile >= p.num_tiles) return;
+    const int r = idx - tile * heads_per_xcd;
+    kvh = xcd * (p.H_kv >> 3) + r / group;
+    hg = r % group;
+  } else {
+    const int w = xcd * per_xcd + idx;
+    if (w >= p.num_tiles * p.H) return;
+    hg = w % group;
+    tile = (w / group) % p.num_tiles;
+    kvh = w / (group * p.num_tiles);
+  }
   const int head = kvh * group + hg;
   int b = 0, q_begin = 0, q_len = 0;
   {
     int tile_in_request = 0;
-    if (!locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request)) return;
+    const bool found = p.B <= 64 ? locate_query_tile_lpt(p.cu_q, p.cu_k, p.B, BM, tile, b, q_begin, q_len, tile_in_request)
+                                 : locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request);
+    if (!found) return;
     tile = tile_in_request;
   }
 
