@@ -25,6 +25,11 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, vendor figure
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 
+# HBM bytes per launch of the default workloads, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (raw counters scaled by what they read for the 1 GiB copy of --copy-calibration: x2.000 and x1.000);
+# the summaries with the commands are profiles/relocate_kernel_*.md and profiles/varlen_attn_dma_kernel_*.md.
+MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 17.991e9, "attention": 260.0e6}
+
 
 def _event_times_ms(fn, steps, torch):
     """Average launch duration in ms: one HIP event pair on the current stream around `steps` back-to-back launches
@@ -118,8 +123,8 @@ def attention_bench(torch, device, ops, steps, warmup):
                                "kv = affix + request + 256 (920-1712), slot map over shared affix slots and shuffled private blocks",
                    "total_q": total_q, "total_kv": sum(w["kv_lens"])},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
-                     "kernel": "varlen_attn_kernel<bf16,128>", "algorithmic_flops": flops,
+                     "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["attention"],
+                     "kernel": "varlen_attn_dma_kernel<bf16,128,plain>", "algorithmic_flops": flops,
                      "algorithmic_bytes": kv_bytes + qo_bytes,
                      "achieved_GBps": round((kv_bytes + qo_bytes) / (avg_ms * 1e-3) / 1e9, 1)},
     }
@@ -202,6 +207,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="layers of the relocation workload (32 = LLaDA-8B)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-attention", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run three plain 1 GiB device copies (known traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--engine", action="store_true", help="run the engine-step sweep (configs[4]) instead")
     ap.add_argument("--engine-layers", type=int, default=32)
     ap.add_argument("--engine-batch", type=int, default=16)
@@ -224,6 +231,14 @@ def main():
         sys.exit(3)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.copy_calibration:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device=device).random_(0, 255)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_calibration": "3 x 1 GiB device-to-device copy_", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return
     if args.engine:
         engine_bench(torch, device, args)
         return
@@ -272,14 +287,15 @@ def main():
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES["relocate_32_layers"] if args.layers == 32 else None,
             "kernel": "relocate_kernel<bf16,128>", "avg_launch_ms": round(avg_kernel_ms, 4),
             "algorithmic_bytes": algo_bytes,
         },
     }
 
     if not args.no_attention:
-        result["attention"] = attention_bench(torch, device, ops, steps=args.steps, warmup=args.warmup)
+        result["attention"] = attention_bench(torch, device, ops, steps=max(args.steps, 20), warmup=args.warmup)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_relocation_baseline(torch, wl)
