@@ -130,6 +130,35 @@ def attention_bench(torch, device, ops, steps, warmup):
     }
 
 
+def attention_shape_sweep(torch, device, ops, steps):
+    """Uniform-shape runs of the same attention kernel (MHA, 32 heads, D = 128, bf16, identity slot map): decode-like
+    shapes are bound by streaming K/V once, long-query shapes by the matrix core.  Median of per-call HIP event pairs."""
+    H, D = 32, 128
+    rows = []
+    for B, q, kv in ((16, 32, 1400), (16, 32, 2800), (64, 32, 1400), (16, 128, 1400), (16, 600, 1400), (4, 4096, 4096)):
+        S = B * kv
+        Q = (torch.randn(B * q, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        K = (torch.randn(S, 1, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        V = (torch.randn(S, 1, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        cu_q = torch.arange(0, (B + 1) * q, q, dtype=torch.int32, device=device)
+        cu_k = torch.arange(0, (B + 1) * kv, kv, dtype=torch.int32, device=device)
+        slots = torch.arange(S, dtype=torch.int32, device=device)
+        for _ in range(3):
+            ops.acache_attention(Q, K, V, cu_q, cu_k, slots)
+        torch.cuda.synchronize()
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for a, b in pairs:
+            a.record()
+            ops.acache_attention(Q, K, V, cu_q, cu_k, slots)
+            b.record()
+        torch.cuda.synchronize()
+        ms = statistics.median(a.elapsed_time(b) for a, b in pairs)
+        kv_bytes = 2 * S * H * D * 2
+        rows.append({"B": B, "q": q, "kv": kv, "us": round(ms * 1e3, 1), "TFLOPs": round(4 * H * D * B * q * kv / ms / 1e9, 0),
+                     "kv_GBps": round(kv_bytes / ms / 1e6, 0)})
+    print(json.dumps({"attention_shape_sweep": rows}))
+
+
 def engine_bench(torch, device, args):
     """configs[4]: nano-vdllm-style engine step on random-init LLaDA-8B-shaped weights, anchor-ratio sweep
     against full affix recompute.  Prints one JSON line of its own (not part of the default run)."""
@@ -209,6 +238,7 @@ def main():
     ap.add_argument("--no-attention", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three plain 1 GiB device copies (known traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--attention-shapes", action="store_true", help="only run the attention kernel on a few uniform shapes")
     ap.add_argument("--engine", action="store_true", help="run the engine-step sweep (configs[4]) instead")
     ap.add_argument("--engine-layers", type=int, default=32)
     ap.add_argument("--engine-batch", type=int, default=16)
@@ -238,6 +268,9 @@ def main():
             b.copy_(a)
         torch.cuda.synchronize()
         print(json.dumps({"copy_calibration": "3 x 1 GiB device-to-device copy_", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return
+    if args.attention_shapes:
+        attention_shape_sweep(torch, device, ops, args.steps)
         return
     if args.engine:
         engine_bench(torch, device, args)
