@@ -15,7 +15,9 @@ the paged engine of this package (``ModelRunner`` + HIP kernels).  Consequences 
   slots.  A per-layer tuple of ``(k, v)`` with the HF layout ``[1, H_kv, A, D]`` and PRE-RoPE keys
   (llada/generate_ACache.py:153) is rotated to positions ``0..A-1`` and scattered into the shared
   slots instead of being recomputed;
-* ``factor`` (dynamic threshold) and ``drop_non_anchor`` are not implemented and raise.
+* ``drop_non_anchor`` is served by leaving the frozen affix rows out of the request's read slot map:
+  anchors and non-affix tokens keep their position ids and never see the dropped tokens
+  (the reference's compact kept-position sequence, llada/generate_ACache.py:478-491).
 """
 from __future__ import annotations
 
@@ -30,6 +32,21 @@ from .model_runner import ModelRunner
 from .ops import select_anchor_tokens  # noqa: F401  (re-exported: same name as the reference)
 from .sequence import Sequence
 from .utils import add_gumbel_noise, reset_context
+
+
+def _coerce_bool(value, default: bool, arg_name: str) -> bool:
+    """``None`` -> default; bools and numbers by truth value; otherwise the usual string spellings
+    (llada/generate_ACache.py:21-35: the evaluation CLI hands strings through)."""
+    if value is None:
+        return default
+    if isinstance(value, (bool, int, float)):
+        return bool(value)
+    text = str(value).strip().lower()
+    if text in ("1", "true", "yes", "y", "on"):
+        return True
+    if text in ("0", "false", "no", "n", "off"):
+        return False
+    raise ValueError(f"{arg_name} must be a boolean-like value, got {value!r}.")
 
 
 def ceil_to_int(value: float) -> int:
@@ -79,6 +96,43 @@ def get_transfer_index(logits, temperature, remasking, mask_index, x, num_transf
     cols = torch.arange(confidence.shape[1], device=confidence.device).unsqueeze(0)
     picked = torch.zeros_like(confidence, dtype=torch.int8).scatter(1, idx, (cols < k.unsqueeze(1)).to(torch.int8))
     return x0, picked.bool() & mask_index
+
+
+def get_transfer_index_dynamic(logits, temperature, remasking, mask_index, x, num_transfer_tokens, factor=1):
+    """Dynamic-threshold transfer (llada/generate.py:379-420).
+
+    Per row, with n masked tokens and their confidences sorted descending c_1 >= ... >= c_n: commit the
+    leading tokens while c_i >= 1 - factor / (i + 1) (the first always passes), stopping at the first
+    failure.  The reference's loop leaves ``top_i`` at the failing index, or at n - 1 when nothing fails, and
+    then adds one when ``top_i`` is 0 or n - 1; both quirks are kept: a row whose only failure is its last
+    token commits all n.  ``num_transfer_tokens`` is ignored, as in the reference.
+    """
+    x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
+    if remasking == "low_confidence":
+        p = F.softmax(logits.to(torch.float64), dim=-1)
+        x0_p = torch.gather(p, dim=-1, index=x0.unsqueeze(-1)).squeeze(-1)
+    elif remasking == "random":
+        x0_p = torch.rand(x0.shape, device=x0.device, dtype=torch.float64)
+    else:
+        raise NotImplementedError(remasking)
+    x0 = torch.where(mask_index, x0, x)
+    confidence = torch.where(mask_index, x0_p, torch.full_like(x0_p, float("-inf")))
+    transfer = torch.zeros_like(x0, dtype=torch.bool)
+    counts = mask_index.sum(dim=1).tolist()
+    ordered, order = torch.sort(confidence, dim=1, descending=True, stable=True)
+    ordered = ordered.tolist()
+    for j, n in enumerate(counts):
+        if n == 0:
+            continue
+        top_i = 0
+        for top_i in range(n):
+            thresh = -1.0 if top_i == 0 else 1.0 - factor / (top_i + 2)
+            if ordered[j][top_i] < thresh:
+                break
+        if top_i == 0 or top_i == n - 1:
+            top_i += 1
+        transfer[j, order[j, :top_i]] = True
+    return x0, transfer
 
 
 # ------------------------------------------------------------------------------------------ engine glue
@@ -190,10 +244,7 @@ def generate_with_anchor_attention(
     """
     B = prompt.shape[0]
     assert B == 1, "generate_with_anchor_attention currently supports batch_size=1."
-    if factor is not None:
-        raise NotImplementedError("dynamic-threshold transfer (factor) is not implemented on the paged engine")
-    if drop_non_anchor:
-        raise NotImplementedError("drop_non_anchor is not implemented on the paged engine")
+    drop_non_anchor = _coerce_bool(drop_non_anchor, default=False, arg_name="drop_non_anchor")
     Lp = int(prompt.shape[1])
     assert gen_length % block_length == 0
     num_blocks = gen_length // block_length
@@ -248,7 +299,9 @@ def generate_with_anchor_attention(
     else:
         anchors = []
     seq.set_anchor_positions(anchors)
-    runner._reserve_single_sequence_relocation_workspace(seq)
+    seq.drop_non_anchor = drop_non_anchor
+    if not drop_non_anchor:  # nothing of the frozen affix is read in the strict ablation: no relocated copy needed
+        runner._reserve_single_sequence_relocation_workspace(seq)
     runner.block_manager.allocate(seq)
     runner._finalize_sequence_layout(seq)
 
@@ -273,9 +326,13 @@ def generate_with_anchor_attention(
                         decoding_positions = runner.prepare_decoding_acache([seq])
                     logits = runner.model(block, position_ids=decoding_positions).logits
                     nfe += 1
-                quota = None if threshold is not None else quotas[:, i]
-                x0, transfer = get_transfer_index(logits, temperature, remasking, block == mask_id, block, quota,
-                                                  threshold)
+                if factor is None:
+                    quota = None if threshold is not None else quotas[:, i]
+                    x0, transfer = get_transfer_index(logits, temperature, remasking, block == mask_id, block, quota,
+                                                      threshold)
+                else:
+                    x0, transfer = get_transfer_index_dynamic(logits, temperature, remasking, block == mask_id, block,
+                                                              None, factor)
                 block = torch.where(transfer, x0, block)
             seq.token_ids[s:s + block_length] = block[0].tolist()
     finally:

@@ -207,6 +207,15 @@ class ModelRunner:
 
     def _attention_read_layout(self, seq, use_query_relocation: bool):
         """Read slots of one request; shared affix slots packed first for query-side relocation (275-282)."""
+        if getattr(seq, "drop_non_anchor", False):
+            # strict ablation of the HF path (llada/generate_ACache.py:478-491): the frozen affix rows are not
+            # read at all; anchors and non-affix tokens live in private slots and keep their position ids
+            slots = np.asarray(seq.read_slot_map, dtype=np.int64)
+            frozen = (slots >= seq.shared_slot_offset) & (slots < seq.shared_slot_offset + self.shared_prefix_len)
+            if self._relocated_affix_slot_offset is not None:
+                lo = self._relocated_affix_slot_offset
+                frozen |= (slots >= lo) & (slots < lo + self.shared_prefix_len)
+            return slots[~frozen].tolist(), 0
         if not use_query_relocation or seq.affix_start == 0:
             return list(seq.read_slot_map), 0
         lo = seq.shared_slot_offset
@@ -606,7 +615,7 @@ class ModelRunner:
             shifts.append(seq.affix_start if self._affix_relocation_enabled else 0)
             block_starts.append(cu_q[-1] + seq.block_query_start())
             cu_q.append(cu_q[-1] + q_pos.size)
-            cu_k.append(cu_k[-1] + len(seq))
+            cu_k.append(cu_k[-1] + len(layout))
         kv_lens = np.diff(cu_k)
         set_context(
             True, self._to_device(cu_q, torch.int32), self._to_device(cu_k, torch.int32),
@@ -635,7 +644,7 @@ class ModelRunner:
             reads.append(np.asarray(layout, dtype=np.int64))
             shared_lens.append(shared_len)
             shifts.append(seq.affix_start if self._affix_relocation_enabled else 0)
-            cu_k.append(cu_k[-1] + len(seq))
+            cu_k.append(cu_k[-1] + len(layout))
         kv_lens = np.diff(cu_k)
         positions = np.asarray(starts, dtype=np.int64)[:, None] + np.arange(block_length)[None, :]
         cu_q = np.arange(len(group) + 1) * block_length

@@ -116,13 +116,43 @@ def test_importance_entry_point_and_anchor_selection(device):
     assert idx.shape == (1, 5) and idx[0].tolist() == sorted(torch.topk(imp[0], 5).indices.tolist())
 
 
-def test_unsupported_flags_raise(device):
+def test_drop_non_anchor_never_sees_the_dropped_affix_tokens(device):
+    """Strict ablation (llada/generate_ACache.py:478-491): with the frozen affix rows left out of attention, the
+    output may depend on the affix only through the anchors.  Ratio 0 keeps no anchor, so two different affixes of
+    the same length must give the same generation; ratio 1 keeps every affix token, so nothing is dropped and the
+    result equals the ordinary path."""
+    cfg, model = _model(device, seed=4)
+    head, tail = [3, 4], [5, 6, 7]
+    args = dict(steps=8, gen_length=8, block_length=4, mask_id=MASK, threshold=0.9, affix_start=2, affix_end=22)
+    outs = []
+    for affix in (list(range(10, 30)), list(range(40, 60))):
+        prompt = torch.tensor([head + affix + tail], device=device)
+        x, nfe = G.generate_with_anchor_attention(model, prompt, anchor_ratio=0.0, drop_non_anchor=True, **args)
+        assert x.shape == (1, prompt.shape[1] + 8) and (x[0, -8:] != MASK).all()
+        outs.append(x[0, -8:].tolist())
+    assert outs[0] == outs[1]
+    prompt = torch.tensor([head + list(range(10, 30)) + tail], device=device)
+    full_drop, _ = G.generate_with_anchor_attention(model, prompt, anchor_ratio=1.0, drop_non_anchor="true", **args)
+    full_keep, _ = G.generate_with_anchor_attention(model, prompt, anchor_ratio=1.0, drop_non_anchor=False, **args)
+    assert full_drop.tolist() == full_keep.tolist()
+
+
+def test_dynamic_threshold_factor_runs_and_bounds_nfe(device):
+    cfg, model = _model(device, seed=5)
+    prompt = torch.tensor([[3, 4] + list(range(10, 30)) + [5, 6]], device=device)
+    x, nfe = G.generate_with_anchor_attention(model, prompt, steps=8, gen_length=8, block_length=4, mask_id=MASK,
+                                              factor=1.0, anchor_ratio=0.25, affix_start=2, affix_end=22)
+    assert (x[0, -8:] != MASK).all()
+    # every step commits at least one token: at most 4 forwards per block of 4, at least 1; plus the importance pass
+    assert 1 + 2 <= nfe <= 1 + 8
+
+
+def test_argument_errors(device):
     cfg, model = _model(device)
     p = torch.tensor([[3, 4, 5, 6]], device=device)
-    with pytest.raises(NotImplementedError):
-        G.generate_with_anchor_attention(model, p, steps=4, gen_length=4, block_length=4, mask_id=MASK, factor=1.0, affix_end=2)
-    with pytest.raises(NotImplementedError):
-        G.generate_with_anchor_attention(model, p, steps=4, gen_length=4, block_length=4, mask_id=MASK, drop_non_anchor=True, affix_end=2)
+    with pytest.raises(ValueError, match="boolean-like"):
+        G.generate_with_anchor_attention(model, p, steps=4, gen_length=4, block_length=4, mask_id=MASK,
+                                         drop_non_anchor="perhaps", affix_end=2)
     with pytest.raises(ValueError, match="must not overlap"):
         G.generate_with_anchor_attention(model, p, steps=2, gen_length=2, block_length=2, mask_id=MASK,
                                          affix_start=0, affix_end=3, generation_start=2)
