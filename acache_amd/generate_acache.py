@@ -14,7 +14,7 @@ the paged engine of this package (``ModelRunner`` + HIP kernels).  Consequences 
 * ``precomputed_affix_cache`` is optional.  ``None``: the affix is encoded once into the shared
   slots.  A per-layer tuple of ``(k, v)`` with the HF layout ``[1, H_kv, A, D]`` and PRE-RoPE keys
   (llada/generate_ACache.py:153) is rotated to positions ``0..A-1`` and scattered into the shared
-  slots instead of being recomputed;
+  slots instead of being recomputed (the Dream layout ``[1, A, H_kv * D]`` is accepted too);
 * ``drop_non_anchor`` is served by leaving the frozen affix rows out of the request's read slot map:
   anchors and non-affix tokens keep their position ids and never see the dropped tokens
   (the reference's compact kept-position sequence, llada/generate_ACache.py:478-491).
@@ -165,9 +165,16 @@ def _ingest_affix_cache(runner: ModelRunner, affix_tokens, affix_cache):
     assert len(affix_cache) == len(blocks), "precomputed_affix_cache must have one (key, value) pair per layer"
     positions = torch.arange(n, device=runner.device)
     slots = torch.arange(n, dtype=torch.int32, device=runner.device)
+    hkv, hd = runner.kv_cache.shape[-2], runner.kv_cache.shape[-1]
     for (k, v), block in zip(affix_cache, blocks):
-        k = k[0].permute(1, 0, 2).contiguous().to(runner.kv_cache.dtype)
-        v = v[0].permute(1, 0, 2).contiguous().to(runner.kv_cache.dtype)
+        if k.dim() == 4:   # LLaDA HF layout [1, H_kv, A, D]
+            k = k[0].permute(1, 0, 2)
+            v = v[0].permute(1, 0, 2)
+        else:              # Dream HF layout [1, A, H_kv * D] (dream/generate_ACache.py:198)
+            k = k[0].view(n, hkv, hd)
+            v = v[0].view(n, hkv, hd)
+        k = k.contiguous().to(runner.kv_cache.dtype)
+        v = v.contiguous().to(runner.kv_cache.dtype)
         if getattr(runner.config.hf_config, "rope", True):
             _, k = block.rotary_emb(k, k, positions, max(n, runner.config.hf_config.max_sequence_length))
         ops.store_kvcache(k.contiguous(), v, block.attn.k_cache, block.attn.v_cache, slots)
@@ -189,7 +196,8 @@ def compute_attention_importance_cross_affix(model, full_input_ids, affix_cache=
     tokens = full_input_ids[0].tolist()
     if affix_len is None:
         assert affix_cache is not None, "affix_len or affix_cache is required"
-        affix_len = affix_cache[0][0].shape[2]
+        sample_k = affix_cache[0][0]
+        affix_len = sample_k.shape[2] if sample_k.dim() == 4 else sample_k.shape[1]
     runner = _as_runner(model, mask_id=mask_id, block_length=1, gen_length=0, anchor_ratio=1.0,
                         selection_mode="top", threshold=None, temperature=0.0, remasking="low_confidence",
                         total_len=len(tokens), affix_len=affix_len)
@@ -242,6 +250,36 @@ def generate_with_anchor_attention(
 
     Returns ``(x, nfe)`` with ``x`` of shape ``(1, prompt_len [+ gen_length])`` like the reference.
     """
+    return _generate(model, prompt, steps, gen_length, block_length, temperature, remasking, mask_id, threshold, factor,
+                     affix_start, affix_end, generation_start, anchor_ratio, selection_mode, drop_non_anchor,
+                     precomputed_affix_cache, dream=False)
+
+
+def sample_tokens(logits, temperature=0.0):
+    """``(confidence, token)`` per row: arg-max of the softmax at temperature 0, a categorical draw from
+    ``softmax(logits / temperature)`` otherwise (dream/model/generation_utils_block.py:80-112 without top-p/top-k)."""
+    if temperature > 0:
+        logits = logits / temperature
+    probs = torch.softmax(logits, dim=-1)
+    if temperature > 0:
+        x0 = torch.distributions.Categorical(probs=probs).sample()
+        return torch.gather(probs, -1, x0.unsqueeze(-1)).squeeze(-1), x0
+    return probs.max(dim=-1)
+
+
+def _shift_right(logits):
+    """Dream alignment (dream/generate_ACache.py:47-49): row i takes the logits of row i - 1, row 0 keeps its own."""
+    return torch.cat([logits[:, :1], logits[:, :-1]], dim=1)
+
+
+@torch.no_grad()
+def _generate(model, prompt, steps, gen_length, block_length, temperature, remasking, mask_id, threshold, factor,
+              affix_start, affix_end, generation_start, anchor_ratio, selection_mode, drop_non_anchor,
+              precomputed_affix_cache, dream: bool):
+    """Shared body of the LLaDA (llada/generate_ACache.py:311-629) and Dream (dream/generate_ACache.py:425-737)
+    entry points.  Dream differs in four places: all-anchor selection skips the importance pass, logits are taken
+    one compact position to the left, a block refresh commits only the block's first token, and the remaining
+    ``steps_per_block - 1`` steps share the quota."""
     B = prompt.shape[0]
     assert B == 1, "generate_with_anchor_attention currently supports batch_size=1."
     drop_non_anchor = _coerce_bool(drop_non_anchor, default=False, arg_name="drop_non_anchor")
@@ -272,10 +310,12 @@ def generate_with_anchor_attention(
             "Generation span must not overlap affix span. "
             f"Got generation=[{gen_start}, {gen_start + gen_length}), affix=[{affix_start}, {affix_end}).")
     affix_len = affix_end - affix_start
-    if precomputed_affix_cache is not None and precomputed_affix_cache[0][0].shape[2] != affix_len:
-        raise ValueError(
-            f"precomputed_affix_cache length {precomputed_affix_cache[0][0].shape[2]} does not match "
-            f"expected affix length {affix_len}.")
+    if precomputed_affix_cache is not None:
+        sample_k = precomputed_affix_cache[0][0]
+        cached_len = sample_k.shape[2] if sample_k.dim() == 4 else sample_k.shape[1]
+        if cached_len != affix_len:
+            raise ValueError(
+                f"precomputed_affix_cache length {cached_len} does not match expected affix length {affix_len}.")
 
     runner = _as_runner(model, mask_id=mask_id, block_length=block_length, gen_length=gen_length,
                         anchor_ratio=anchor_ratio, selection_mode=selection_mode, threshold=threshold,
@@ -290,7 +330,9 @@ def generate_with_anchor_attention(
     k = min(ceil_to_int(anchor_ratio * affix_len), affix_len)
     seq.enable_acache(affix_len, anchor_ratio, affix_start=affix_start, affix_end=affix_end)
     assert seq.num_anchor_tokens == k
-    if k > 0:
+    if dream and k >= affix_len and affix_len > 0:
+        anchors = list(range(affix_start, affix_end))   # every affix token is an anchor: nothing to rank
+    elif k > 0:
         if selection_mode == "random":
             anchors = (torch.randperm(affix_len, device=device)[:k].sort().values + affix_start).tolist()
         else:
@@ -315,19 +357,29 @@ def generate_with_anchor_attention(
             # block boundary: recompute anchors + every non-affix token against the frozen affix
             input_ids, positions, block_starts = runner.prepare_caching_acache([seq])
             keep = (block_starts.unsqueeze(1) + offsets).flatten().long()
+            if dream:  # logits of the compact position to the left (the first compact row keeps its own)
+                keep = (keep - 1).clamp_(min=0)
             logits = runner.model(input_ids, position_ids=positions, logits_keep_indices=keep).logits.unsqueeze(0)
             nfe += 1
             decoding_positions = None
-            for i in range(steps_per_block):
+            if dream:
+                # commit only the block's first token, then share the quota over the remaining steps
+                _, seed = sample_tokens(logits, temperature=temperature)
+                block[:, 0] = seed[:, 0]
+                quotas = (get_num_transfer_tokens(block == mask_id, steps_per_block - 1)
+                          if factor is None and threshold is None and steps_per_block > 1 else None)
+            for i in range(1 if dream else 0, steps_per_block):
                 if i > 0:
                     if (block == mask_id).sum() == 0:
                         break
                     if decoding_positions is None:
                         decoding_positions = runner.prepare_decoding_acache([seq])
                     logits = runner.model(block, position_ids=decoding_positions).logits
+                    if dream:
+                        logits = _shift_right(logits)
                     nfe += 1
                 if factor is None:
-                    quota = None if threshold is not None else quotas[:, i]
+                    quota = None if threshold is not None else quotas[:, i - 1 if dream else i]
                     x0, transfer = get_transfer_index(logits, temperature, remasking, block == mask_id, block, quota,
                                                       threshold)
                 else:

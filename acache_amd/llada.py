@@ -41,6 +41,7 @@ class LLaDAConfig:
     rms_norm_eps: float = 1e-5
     mask_token_id: int = 126336
     weight_tying: bool = False
+    qkv_bias: bool = False  # Dream / Qwen2-style attention projections carry a bias
 
     @property
     def effective_n_kv_heads(self) -> int:
@@ -96,9 +97,9 @@ class LLaDABlock(nn.Module):
         self.head_dim = d // h
         self.attn_norm = RMSNorm(d, config.rms_norm_eps)
         self.ff_norm = RMSNorm(d, config.rms_norm_eps)
-        self.q_proj = nn.Linear(d, h * self.head_dim, bias=False)
-        self.k_proj = nn.Linear(d, hkv * self.head_dim, bias=False)
-        self.v_proj = nn.Linear(d, hkv * self.head_dim, bias=False)
+        self.q_proj = nn.Linear(d, h * self.head_dim, bias=config.qkv_bias)
+        self.k_proj = nn.Linear(d, hkv * self.head_dim, bias=config.qkv_bias)
+        self.v_proj = nn.Linear(d, hkv * self.head_dim, bias=config.qkv_bias)
         self.attn_out = nn.Linear(h * self.head_dim, d, bias=False)
         self.ff_proj = nn.Linear(d, config.mlp_hidden_size, bias=False)
         self.up_proj = nn.Linear(d, config.mlp_hidden_size, bias=False)
@@ -154,8 +155,8 @@ class LLaDAModelLM(nn.Module):
         super().__init__()
         self.config = config
         self.model = LLaDAModel(config)
-        for p in self.parameters():
-            if p.dim() > 1:
+        for name, p in self.named_parameters():
+            if p.dim() > 1 or name.endswith("_proj.bias"):  # norm weights stay at one
                 nn.init.normal_(p, mean=0.0, std=init_std)
 
     @property
