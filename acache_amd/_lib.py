@@ -29,6 +29,10 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         c_int64, c_int32, c_int32, c_int32, c_int32, c_int64,
         c_int64, c_int64, c_int64, c_int64, c_void_p]),
+    "acache_rope_qk_scatter": (c_int32, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        c_int32, c_int64, c_int32, c_int32, c_int32, c_int32, c_int64,
+        c_int64, c_int64, c_int64, c_void_p]),
     "acache_topk_anchors": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "acache_block_table_slots": (c_int32, [

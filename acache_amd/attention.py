@@ -34,7 +34,9 @@ class Attention(nn.Module):
         # patches forward for the same purpose)
         self.probe = None
 
-    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+    def forward(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, kv_stored: bool = False):
+        """``kv_stored``: the caller has already written ``k`` / ``v`` to ``context.slot_mapping`` (the fused
+        rotary + scatter launch); everything else is the reference's ``forward(q, k, v)``."""
         context = get_context()
         k_cache, v_cache = self.k_cache, self.v_cache
         assert k_cache.numel() and v_cache.numel()
@@ -43,7 +45,8 @@ class Attention(nn.Module):
             bs, seqlen = k.shape[:2]
             k = k.reshape(bs * seqlen, self.num_kv_heads, self.head_dim)
             v = v.reshape(bs * seqlen, self.num_kv_heads, self.head_dim)
-        ops.store_kvcache(k, v, k_cache, v_cache, context.slot_mapping)
+        if not kv_stored:
+            ops.store_kvcache(k, v, k_cache, v_cache, context.slot_mapping)
         if self.probe is not None:
             self.probe(self, q)
         scale = self.scale if self.scale is not None else self.head_dim ** -0.5

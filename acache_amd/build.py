@@ -27,6 +27,7 @@ HIP_FLAGS = [
 PER_FILE_FLAGS = {
     # the RoPE rotation must not be contracted into fused multiply-adds
     "relocate.hip": ["-ffp-contract=off"],
+    "rope_scatter.hip": ["-ffp-contract=off"],
 }
 
 

@@ -23,7 +23,9 @@ import torch
 from torch import nn
 import torch.nn.functional as F
 
+from . import ops
 from .attention import Attention
+from .utils import get_context
 from .rope import rope_table
 
 
@@ -55,9 +57,8 @@ class RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
-        xf = x.float()
-        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)
-        return (xf * self.weight.float()).to(x.dtype)
+        # one fused kernel; statistics and scaling in fp32, one rounding to the activation type
+        return F.rms_norm(x, (x.shape[-1],), self.weight.to(x.dtype), self.eps)
 
 
 class RotaryEmbedding(nn.Module):
@@ -114,9 +115,17 @@ class LLaDABlock(nn.Module):
         q = self.q_proj(y).view(*lead, h, hd)
         k = self.k_proj(y).view(*lead, hkv, hd)
         v = self.v_proj(y).view(*lead, hkv, hd)
-        if self.config.rope:
-            q, k = self.rotary_emb(q, k, position_ids, max_pos)
-        o = self.attn(q, k, v)
+        if self.config.rope and q.is_cuda:
+            # rotary application and the K/V cache write in one launch (q and k are rotated in place)
+            sin, cos = self.rotary_emb.get_rotary_embedding(max_pos or self.config.max_sequence_length, q.device)
+            ops.rope_qk_scatter(q.view(-1, h, hd), k.view(-1, hkv, hd), v.view(-1, hkv, hd),
+                                position_ids.reshape(-1).contiguous(), cos, sin,
+                                self.attn.k_cache, self.attn.v_cache, get_context().slot_mapping)
+            o = self.attn(q, k, v, kv_stored=True)
+        else:
+            if self.config.rope:
+                q, k = self.rotary_emb(q, k, position_ids, max_pos)
+            o = self.attn(q, k, v)
         x = x + self.attn_out(o.reshape(*lead, h * hd))
         y = self.ff_norm(x)
         return x + self.ff_out(F.silu(self.ff_proj(y)) * self.up_proj(y))

@@ -196,6 +196,51 @@ def store_kvcache(
     _lib.check(rc, "store_kvcache")
 
 
+def rope_qk_scatter(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor | None,
+    positions: torch.Tensor,
+    rope_cos: torch.Tensor,
+    rope_sin: torch.Tensor,
+    k_cache: torch.Tensor | None = None,
+    v_cache: torch.Tensor | None = None,
+    slot_mapping: torch.Tensor | None = None,
+):
+    """Rotate ``q`` and ``k`` in place to their positions and write ``k`` / ``v`` to their cache slots, one launch.
+
+    ``q``: ``[N, H, D]``, ``k`` / ``v``: ``[N, H_kv, D]`` (token stride free, heads contiguous: views of a fused
+    projection are fine); ``positions``: int64 ``[N]``; tables fp32 ``[rows, D]``.  Without ``slot_mapping`` only
+    the rotation is done.  Rotary application of nano-vdllm/model/modeling_llada.py:412-453 followed by
+    ``store_kvcache`` (nano-vdllm/model/attention.py:34-41).
+    """
+    N, H, D = q.shape
+    H_kv = k.shape[1]
+    assert k.shape == (N, H_kv, D) and q.is_cuda and q.dtype == k.dtype
+    assert q.stride(-1) == 1 and k.stride(-1) == 1 and q.stride(1) == D and k.stride(1) == D
+    assert positions.dtype == torch.int64 and positions.numel() == N and positions.is_contiguous()
+    assert rope_cos.dtype == torch.float32 and rope_cos.is_contiguous() and rope_cos.shape[1] == D
+    assert rope_sin.dtype == torch.float32 and rope_sin.is_contiguous() and rope_sin.shape == rope_cos.shape
+    slots = None
+    num_slots = 0
+    if slot_mapping is not None:
+        assert v is not None and k_cache is not None and v_cache is not None
+        assert v.shape == k.shape and v.stride(-1) == 1 and v.stride(1) == D and v.dtype == q.dtype
+        assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == q.dtype == v_cache.dtype
+        assert slot_mapping.numel() == N
+        slots = _i32(slot_mapping, "slot_mapping")
+        num_slots = k_cache.numel() // (H_kv * D)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        rc = lib.acache_rope_qk_scatter(
+            _ptr(q), _ptr(k), _ptr(v) if slots is not None else None,
+            _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None,
+            _ptr(positions), _ptr(slots) if slots is not None else None, _ptr(rope_cos), _ptr(rope_sin),
+            rope_cos.shape[0], N, H, H_kv, D, _code(q), num_slots,
+            q.stride(0), k.stride(0), v.stride(0) if slots is not None else 0, _stream(q))
+    _lib.check(rc, "rope_qk_scatter")
+
+
 def kv_scatter_layers(
     key: torch.Tensor,
     value: torch.Tensor,

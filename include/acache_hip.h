@@ -129,6 +129,38 @@ int acache_kv_scatter(
     void *stream);
 
 /*
+ * RoPE on freshly projected q / k rows, fused with the scatter of k / v into the
+ * paged cache of one layer: the step in front of attention.
+ *
+ *   for i < N, with p = positions[i]:
+ *     q[i, h, :]  = rope(q[i, h, :], p)            for h < H      (in place)
+ *     k[i, h, :]  = rope(k[i, h, :], p)            for h < H_kv   (in place)
+ *     if slot_map[i] >= 0:
+ *       k_cache[slot_map[i], :, :] = k[i, :, :]   (the rotated rows)
+ *       v_cache[slot_map[i], :, :] = v[i, :, :]
+ *   rope(x, p) = x * cos[p] + rot_half(x) * sin[p] in fp32, products and sum
+ *   rounded separately, one rounding to `dtype`.
+ *
+ * Replaces the rotary application of the model's attention block
+ * (nano-vdllm/model/modeling_llada.py:412-453: q and k up-cast, rotated with the
+ * cat(freqs, freqs) tables at the given position ids, cast back) followed by
+ * store_kvcache (nano-vdllm/model/attention.py:34-41, called at line 72); one
+ * launch instead of the reference's elementwise chain plus the scatter kernel.
+ *
+ * slot_map may be NULL (no cache write; v and the caches are then unused).  A slot
+ * outside [0, num_slots) is skipped like -1; a position outside [0, rope_rows)
+ * leaves the row unrotated.  q / k / v: [N, heads, D] with the given token
+ * strides (heads contiguous, so the three may be views of one fused projection).
+ */
+int acache_rope_qk_scatter(
+    void *q, void *k, const void *v, void *k_cache, void *v_cache,
+    const int64_t *positions, const int32_t *slot_map,
+    const float *rope_cos, const float *rope_sin, int32_t rope_rows,
+    int64_t N, int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
+    void *stream);
+
+/*
  * Per-request top-k anchor selection over ragged fp32 influence scores.
  *
  *   request b owns scores[cu_affix[b] .. cu_affix[b+1]) and selects

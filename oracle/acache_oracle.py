@@ -74,6 +74,21 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     return (x * cos[:, None, :] + rot_half(x) * sin[:, None, :]).to(x.dtype)
 
 
+def rope_qk_scatter(q, k, v, positions, cos, sin, k_cache=None, v_cache=None, slot_mapping=None):
+    """RoPE at ``positions`` on q and k, then scatter of the rotated k and of v (fused step in front of attention).
+
+    Composition of ``apply_rope`` (rotary application of nano-vdllm/model/modeling_llada.py:412-453: fp32
+    ``x*cos + rot_half(x)*sin`` with the table rows of the position ids, cast back) and ``store_kvcache``
+    (nano-vdllm/model/attention.py:22-41).  Returns the rotated ``(q, k)``; the caches are updated in place.
+    """
+    idx = positions.long()
+    q_rot = apply_rope(q, cos[idx], sin[idx])
+    k_rot = apply_rope(k, cos[idx], sin[idx])
+    if slot_mapping is not None:
+        store_kvcache(k_rot, v, k_cache, v_cache, slot_mapping)
+    return q_rot, k_rot
+
+
 def rotate(x: torch.Tensor, delta: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     """Rotate rows ``x[t]`` (``[T, H, D]``) by signed per-row position shifts ``delta[t]``.
 
