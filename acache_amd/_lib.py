@@ -35,6 +35,8 @@ SIGNATURES = {
         c_int64, c_int64, c_int64, c_void_p]),
     "acache_topk_anchors": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
+    "acache_argmax_confidence": (c_int32, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p]),
     "acache_block_table_slots": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64, c_void_p]),
     "acache_varlen_attn": (c_int32, [

@@ -831,8 +831,17 @@ class ModelRunner:
     # ------------------------------------------------------------------ token transfer (2279-2314)
     def get_transfer_index(self, logits, temperature, remasking, mask_index, x, threshold=0.9):
         """Pick the tokens to commit: confidence >= threshold among masked positions, at least one per row."""
-        x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
-        if remasking == "low_confidence":
+        fused = (logits.is_cuda and logits.stride(-1) == 1 and logits.data_ptr() % 16 == 0
+                 and (logits.shape[-1] * logits.element_size()) % 16 == 0 and logits.is_contiguous())
+        if remasking == "low_confidence" and fused:
+            # one streaming pass per row: arg-max token and exp(logit - logsumexp) together
+            if temperature == 0:
+                x0, x0_p = ops.argmax_confidence(logits)
+            else:
+                x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
+                _, x0_p = ops.argmax_confidence(logits, picks=x0)
+        elif remasking == "low_confidence":
+            x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
             flat = logits.reshape(-1, logits.shape[-1])
             picks = x0.reshape(-1)
             conf = torch.empty(picks.shape, dtype=torch.float32, device=logits.device)
@@ -842,6 +851,7 @@ class ModelRunner:
                 conf[lo:lo + 64] = torch.exp(chosen - torch.logsumexp(rows, dim=-1))
             x0_p = conf.view_as(x0)
         elif remasking == "random":
+            x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
             x0_p = torch.rand(x0.shape, device=x0.device)
         else:
             raise NotImplementedError(remasking)

@@ -241,6 +241,31 @@ def rope_qk_scatter(
     _lib.check(rc, "rope_qk_scatter")
 
 
+def argmax_confidence(logits: torch.Tensor, picks: torch.Tensor | None = None):
+    """``(token, confidence)`` per row of ``logits`` (``[..., V]``): the arg-max token (or ``picks``) and
+    ``exp(logit[token] - logsumexp(row))`` in fp32, one streaming pass per row
+    (nano-vdllm/model_runner.py:2279-2296)."""
+    V = logits.shape[-1]
+    flat = logits.reshape(-1, V)
+    assert flat.is_cuda and flat.stride(-1) == 1
+    R = flat.shape[0]
+    conf = torch.empty(R, dtype=torch.float32, device=logits.device)
+    if picks is None:
+        token = torch.empty(R, dtype=torch.int64, device=logits.device)
+        picks_flat = None
+    else:
+        picks_flat = picks.reshape(-1).to(torch.int64).contiguous()
+        assert picks_flat.numel() == R
+        token = picks_flat
+    lib = _lib.load()
+    with torch.cuda.device(logits.device):
+        rc = lib.acache_argmax_confidence(
+            _ptr(token) if picks is None else None, _ptr(conf), _ptr(flat), _ptr(picks_flat) if picks is not None else None,
+            R, V, flat.stride(0) if R > 1 else max(V, flat.stride(0)), _code(flat), _stream(flat))
+    _lib.check(rc, "argmax_confidence")
+    return token.view(logits.shape[:-1]), conf.view(logits.shape[:-1])
+
+
 def kv_scatter_layers(
     key: torch.Tensor,
     value: torch.Tensor,

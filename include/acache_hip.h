@@ -184,6 +184,25 @@ int acache_topk_anchors(
     void *stream);
 
 /*
+ * Proposed token and its confidence per logits row (masked-diffusion transfer rule).
+ *
+ *   for r < R:
+ *     t = picks ? picks[r] : argmax_v logits[r, v]          (first maximum)
+ *     out_token[r] = t
+ *     out_conf[r]  = exp(logits[r, t] - logsumexp_v logits[r, v])    in fp32
+ *
+ * Replaces the per-64-row loop of get_transfer_index
+ * (nano-vdllm/model_runner.py:2279-2296: up-cast to fp32, gather of the chosen
+ * logit, torch.logsumexp, exp) and the arg-max in front of it at temperature 0;
+ * with temperature > 0 the caller draws the Gumbel arg-max itself and passes it
+ * as `picks` (out_token may then be NULL).  The row is read once.  Logits are
+ * assumed free of NaN.  row_stride in elements, a multiple of 16 bytes.
+ */
+int acache_argmax_confidence(
+    int64_t *out_token, float *out_conf, const void *logits, const int64_t *picks,
+    int64_t R, int64_t V, int64_t row_stride, int32_t dtype, void *stream);
+
+/*
  * Expand per-request block tables into a flat slot map.
  *
  *   out_slots[cu_k[b] + n] = block_tables[b, n / block_size] * block_size + n % block_size

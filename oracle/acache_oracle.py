@@ -89,6 +89,16 @@ def rope_qk_scatter(q, k, v, positions, cos, sin, k_cache=None, v_cache=None, sl
     return q_rot, k_rot
 
 
+def argmax_confidence(logits, picks=None):
+    """Token and confidence of the transfer rule, nano-vdllm/model_runner.py:2279-2296: ``x0 = argmax`` (or the
+    given picks) and ``exp(logit[x0] - logsumexp(row))`` on the fp32 up-cast."""
+    rows = logits.reshape(-1, logits.shape[-1]).float()
+    x0 = rows.argmax(dim=-1) if picks is None else picks.reshape(-1).long()
+    chosen = rows.gather(-1, x0[:, None]).squeeze(-1)
+    conf = torch.exp(chosen - torch.logsumexp(rows, dim=-1))
+    return x0.view(logits.shape[:-1]), conf.view(logits.shape[:-1])
+
+
 def rotate(x: torch.Tensor, delta: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     """Rotate rows ``x[t]`` (``[T, H, D]``) by signed per-row position shifts ``delta[t]``.
 
