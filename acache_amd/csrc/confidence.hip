@@ -1,10 +1,11 @@
 // Token proposal and its confidence for masked-diffusion decoding (gfx950): per logits row the arg-max
 // token and exp(logit[token] - logsumexp(row)), in one streaming pass over the vocabulary.
 //
-// One 256-thread block per row.  A thread walks 16-byte chunks of the row (stride 256 chunks) keeping an
-// online (max, first index of the max, sum of exp(x - max)) triple in fp32; the triples are merged across
-// the wave with shuffles and across the four waves through LDS.  The row is read once (the torch
-// formulation up-casts it to fp32, gathers, and reduces it twice); bound: HBM, V * bytes per row.
+// One 1024-thread block per row.  A thread walks 16-byte chunks of the row (stride 1024 chunks, four loads
+// in flight) keeping an online (max, first index of the max, sum of exp(x - max)) triple in fp32; the
+// triples are merged across the wave with shuffles and across the sixteen waves through LDS.  The row is
+// read once (the torch formulation up-casts it to fp32, gathers, and reduces it twice); bound: HBM,
+// V * bytes per row.
 #include "common.h"
 
 namespace acache {
@@ -41,8 +42,10 @@ __device__ __forceinline__ RowStat merge(const RowStat &a, const RowStat &b) {
   return r;
 }
 
+constexpr int kConfThreads = 1024;
+
 template <int DTYPE>
-__global__ __launch_bounds__(256) void confidence_kernel(ConfidenceParams p) {
+__global__ __launch_bounds__(kConfThreads) void confidence_kernel(ConfidenceParams p) {
   using E = Elem<DTYPE>;
   constexpr int VEC = E::kPerVec;
   const int tid = threadIdx.x;
@@ -66,7 +69,19 @@ __global__ __launch_bounds__(256) void confidence_kernel(ConfidenceParams p) {
   };
 
   const int64_t full = p.V / VEC;
-  for (int64_t c = tid; c < full; c += 256) {
+  int64_t c = tid;
+  for (; c + 3 * kConfThreads < full; c += 4 * kConfThreads) {  // four independent loads before any use
+    vec16 raw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) raw[u] = load16_stream(row + (c + u * kConfThreads) * 16);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float x[VEC];
+      E::unpack(raw[u], x);
+      take(x, VEC, (c + u * kConfThreads) * VEC);
+    }
+  }
+  for (; c < full; c += kConfThreads) {
     float x[VEC];
     E::unpack(load16_stream(row + c * 16), x);
     take(x, VEC, c * VEC);
@@ -86,13 +101,14 @@ __global__ __launch_bounds__(256) void confidence_kernel(ConfidenceParams p) {
     o.idx = __shfl_xor((long long)st.idx, d);
     st = merge(st, o);
   }
-  __shared__ float sm[4], ss[4];
-  __shared__ long long si[4];
+  constexpr int WAVES = kConfThreads / 64;
+  __shared__ float sm[WAVES], ss[WAVES];
+  __shared__ long long si[WAVES];
   if ((tid & 63) == 0) { sm[tid >> 6] = st.m; ss[tid >> 6] = st.s; si[tid >> 6] = st.idx; }
   __syncthreads();
   if (tid == 0) {
     RowStat r{sm[0], ss[0], si[0]};
-    for (int w = 1; w < 4; ++w) r = merge(r, RowStat{sm[w], ss[w], si[w]});
+    for (int w = 1; w < WAVES; ++w) r = merge(r, RowStat{sm[w], ss[w], si[w]});
     float chosen = r.m;
     if (p.picks) {
       const int64_t pick = p.picks[blockIdx.x];
@@ -126,8 +142,8 @@ extern "C" int acache_argmax_confidence(
   p.out_token = out_token; p.out_conf = out_conf; p.logits = (const char *)logits; p.picks = picks;
   p.V = V; p.row_bytes = row_stride * es;
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == ACACHE_BF16) hipLaunchKernelGGL((confidence_kernel<ACACHE_BF16>), dim3((unsigned)R), dim3(256), 0, s, p);
-  else if (dtype == ACACHE_F16) hipLaunchKernelGGL((confidence_kernel<ACACHE_F16>), dim3((unsigned)R), dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((confidence_kernel<ACACHE_F32>), dim3((unsigned)R), dim3(256), 0, s, p);
+  if (dtype == ACACHE_BF16) hipLaunchKernelGGL((confidence_kernel<ACACHE_BF16>), dim3((unsigned)R), dim3(kConfThreads), 0, s, p);
+  else if (dtype == ACACHE_F16) hipLaunchKernelGGL((confidence_kernel<ACACHE_F16>), dim3((unsigned)R), dim3(kConfThreads), 0, s, p);
+  else hipLaunchKernelGGL((confidence_kernel<ACACHE_F32>), dim3((unsigned)R), dim3(kConfThreads), 0, s, p);
   return launch_status("confidence_kernel");
 }

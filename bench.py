@@ -159,6 +159,83 @@ def attention_shape_sweep(torch, device, ops, steps):
     print(json.dumps({"attention_shape_sweep": rows}))
 
 
+def kernel_sweep(torch, device, ops, steps):
+    """Every other kernel of the path at the shape its config names, plus a plain device copy as the practical HBM
+    reference.  Median of per-call HIP event pairs; bytes are the algorithmic ones."""
+    from acache_amd.rope import rope_table
+    from acache_amd.synthetic import anchor_batch
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for a, b in pairs:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return statistics.median(a.elapsed_time(b) for a, b in pairs) * 1e3  # us
+
+    out = []
+
+    def row(name, us, nbytes, note):
+        out.append({"kernel": name, "us": round(us, 1), "GBps": round(nbytes / us / 1e3, 1), "bytes": nbytes, "workload": note})
+
+    src = torch.empty(1 << 32, dtype=torch.uint8, device=device).random_(0, 255)
+    dst = torch.empty_like(src)
+    row("device copy (torch copy_)", timed(lambda: dst.copy_(src)), 2 * (1 << 32), "4 GiB read + 4 GiB written")
+    del src, dst
+
+    # configs[2]: Dream shape (28 layers, 4 KV heads, D 128), anchors of 16 requests
+    w = anchor_batch(seed=0)
+    L, Hkv, D, BS = 28, 4, 128, 256
+    n_anchor = sum(w["K"])
+    gen = torch.Generator(device=device).manual_seed(0)
+    nblk = sum(-(-k // BS) for k in w["K"]) + 2
+    key = torch.randn(L, n_anchor, Hkv, D, generator=gen, device=device).to(torch.bfloat16)
+    val = torch.randn(L, n_anchor, Hkv, D, generator=gen, device=device).to(torch.bfloat16)
+    kc = torch.zeros(L, nblk, BS, Hkv, D, dtype=torch.bfloat16, device=device)
+    vc = torch.zeros_like(kc)
+    slots = torch.randperm(nblk * BS, device=device)[:n_anchor].to(torch.int32)
+    row("scatter_kernel (all layers, one launch)", timed(lambda: ops.kv_scatter_layers(key, val, kc, vc, slots)),
+        2 * 2 * n_anchor * Hkv * D * 2 * L, f"configs[2]: {n_anchor} anchor rows x 28 layers x 4 KV heads x 128, bf16")
+    scores = torch.cat(w["scores"]).to(device)
+    cu_a = torch.tensor([0] + list(np_cumsum(w["A"])), dtype=torch.int32, device=device)
+    cu_k = torch.tensor([0] + list(np_cumsum(w["K"])), dtype=torch.int32, device=device)
+    starts = torch.tensor(w["affix_start"], dtype=torch.int32, device=device)
+    row("topk_kernel (batch of 16, one launch)", timed(lambda: ops.topk_anchors(scores, cu_a, cu_k, n_anchor, offsets=starts)),
+        4 * sum(w["A"]) + 8 * n_anchor, f"configs[2]: {sum(w['A'])} fp32 scores, {n_anchor} indices out")
+    del key, val, kc, vc
+
+    # the steps on either side of attention, LLaDA-8B shape
+    H, D = 32, 128
+    cos, sin = rope_table(4096, D, 5e5)
+    cos, sin = cos.to(device), sin.to(device)
+    for n_tok, what in ((512, "refinement step: 16 x 32 tokens"), (21252, "block refresh: all tokens of 16 requests")):
+        q = torch.randn(n_tok, H, D, generator=gen, device=device).to(torch.bfloat16)
+        k = torch.randn(n_tok, H, D, generator=gen, device=device).to(torch.bfloat16)
+        v = torch.randn(n_tok, H, D, generator=gen, device=device).to(torch.bfloat16)
+        pos = torch.randint(0, 4096, (n_tok,), generator=gen, device=device)
+        kc = torch.zeros(-(-n_tok // 256) + 1, 256, H, D, dtype=torch.bfloat16, device=device)
+        vc = torch.zeros_like(kc)
+        sl = torch.randperm(kc.shape[0] * 256, device=device)[:n_tok].to(torch.int32)
+        row("rope_scatter_kernel", timed(lambda: ops.rope_qk_scatter(q, k, v, pos, cos, sin, kc, vc, sl)),
+            n_tok * H * D * 2 * (3 + 4), f"{what}, 32 heads x 128, bf16 (q, k, v read; q, k, K-slot, V-slot written)")
+    logits = torch.randn(512, 126464, generator=gen, device=device).to(torch.bfloat16)
+    row("confidence_kernel", timed(lambda: ops.argmax_confidence(logits)), 512 * 126464 * 2,
+        "512 rows x 126 464 logits, bf16")
+    print(json.dumps({"kernel_sweep": out}))
+
+
+def np_cumsum(values):
+    total, acc = 0, []
+    for v in values:
+        total += int(v)
+        acc.append(total)
+    return acc
+
+
 def engine_bench(torch, device, args):
     """configs[4]: nano-vdllm-style engine step on random-init LLaDA-8B-shaped weights, anchor-ratio sweep
     against full affix recompute.  Prints one JSON line of its own (not part of the default run)."""
@@ -239,6 +316,7 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three plain 1 GiB device copies (known traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--attention-shapes", action="store_true", help="only run the attention kernel on a few uniform shapes")
+    ap.add_argument("--kernels", action="store_true", help="only time the other kernels of the path and a plain device copy")
     ap.add_argument("--engine", action="store_true", help="run the engine-step sweep (configs[4]) instead")
     ap.add_argument("--engine-layers", type=int, default=32)
     ap.add_argument("--engine-batch", type=int, default=16)
@@ -271,6 +349,9 @@ def main():
         return
     if args.attention_shapes:
         attention_shape_sweep(torch, device, ops, args.steps)
+        return
+    if args.kernels:
+        kernel_sweep(torch, device, ops, args.steps)
         return
     if args.engine:
         engine_bench(torch, device, args)
