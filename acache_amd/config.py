@@ -36,3 +36,6 @@ class Config:
     acache_memory_reserve_gb: float = 4.0
     profile_timing: bool = False
     model_type: str = "llada"
+    # not in the reference: replay the block-refinement forward from a captured HIP graph (same kernels, same
+    # results, no per-launch host cost); re-captured whenever the attention metadata of the step changes
+    decode_hip_graph: bool = False

@@ -54,6 +54,7 @@ class ModelRunner:
         self._relocated_affix_slot_offset = None
         self.profile_timing = bool(getattr(config, "profile_timing", False))
         self.last_timing = {}
+        self._decode_graph_warm = set()
         self._active_timing = None
         self.allocate_kv_cache()
 
@@ -757,6 +758,7 @@ class ModelRunner:
         last_active = None
         refreshed = adjusted = False
         decoding_positions = None
+        decode_graph = None
         while batch:
             has_mask = (working == mask_id).any(dim=1)
             done = ~has_mask
@@ -806,9 +808,18 @@ class ModelRunner:
                     start = self._start_timing()
                     decoding_positions = (self.prepare_decoding_acache if use_acache else self.prepare_decoding)(
                         batch, active)
+                    decode_graph = None  # new slot maps and positions: the captured launches are stale
                     self._finish_timing(timing, "decode_prepare", start)
                 start = self._start_timing()
-                logits = model(working[active], position_ids=decoding_positions).logits
+                if cfg.decode_hip_graph:
+                    if decode_graph is None:
+                        decode_graph = self._capture_decode_graph(working[active], decoding_positions)
+                        self._add_timing_count(timing, "decode_graph_captures", 1)
+                    graph, graph_tokens, logits = decode_graph
+                    graph_tokens.copy_(working[active])
+                    graph.replay()
+                else:
+                    logits = model(working[active], position_ids=decoding_positions).logits
                 self._finish_timing(timing, "decode_forward", start)
                 self._add_timing_count(timing, "decode_forward_calls", 1)
                 self._add_timing_count(timing, "decode_forward_nfe", len(active))
@@ -827,6 +838,27 @@ class ModelRunner:
             timing["total_nfe"] = int(total_nfe)
         self._active_timing = previous
         return results, total_nfe
+
+    def _capture_decode_graph(self, tokens, positions):
+        """Record one block-refinement forward (``tokens`` ``[n, block_length]`` at ``positions``, attention
+        metadata from the current ``Context``) into a HIP graph.  Returns ``(graph, token buffer, logits buffer)``:
+        copy the step's tokens into the buffer, replay, read the logits.  Every launch of the forward — library
+        GEMMs, the fused rotary + scatter, attention — is recorded from the stream it is enqueued on; nothing in
+        it synchronises with the host.  The first forward of a new shape runs eagerly on a side stream first so
+        that library handles and workspaces exist before the capture."""
+        static_tokens = tokens.clone()
+        shape = (tuple(tokens.shape), len(self._llada_blocks()))
+        if shape not in self._decode_graph_warm:
+            side = torch.cuda.Stream(device=self.device)
+            side.wait_stream(torch.cuda.current_stream(self.device))
+            with torch.cuda.stream(side):
+                self.model(static_tokens, position_ids=positions)
+            torch.cuda.current_stream(self.device).wait_stream(side)
+            self._decode_graph_warm.add(shape)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model(static_tokens, position_ids=positions).logits
+        return graph, static_tokens, logits
 
     # ------------------------------------------------------------------ token transfer (2279-2314)
     def get_transfer_index(self, logits, temperature, remasking, mask_index, x, threshold=0.9):

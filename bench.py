@@ -275,7 +275,7 @@ def engine_bench(torch, device, args):
         return Config(hf_config=cfg, mask_id=cfg.mask_token_id, recompute_batch_size=4, max_num_seqs=0,
                       gen_length=gen, block_length=block, threshold=0.9, cache_block_size=256,
                       num_kvcache_blocks=args.engine_kv_blocks, temperature=0.0, enable_acache=enable,
-                      anchor_ratio=ratio, profile_timing=True)
+                      anchor_ratio=ratio, profile_timing=True, decode_hip_graph=args.engine_graph)
 
     rows = []
     for label, enable, ratio in [("full_recompute", False, 0.0)] + [(f"acache_{r}", True, r) for r in args.engine_ratios]:
@@ -318,6 +318,8 @@ def main():
     ap.add_argument("--attention-shapes", action="store_true", help="only run the attention kernel on a few uniform shapes")
     ap.add_argument("--kernels", action="store_true", help="only time the other kernels of the path and a plain device copy")
     ap.add_argument("--engine", action="store_true", help="run the engine-step sweep (configs[4]) instead")
+    ap.add_argument("--engine-graph", action="store_true",
+                    help="replay the refinement forward from a captured HIP graph (measured: no gain, the loop is GPU-bound)")
     ap.add_argument("--engine-layers", type=int, default=32)
     ap.add_argument("--engine-batch", type=int, default=16)
     ap.add_argument("--engine-affix", type=int, default=1000)

@@ -202,3 +202,33 @@ def test_generate_batched_threshold_loop_matches_dual_cache_token_counts(device,
     if ratio == 1.0:
         agree = sum(a == b for g, h in zip(out, out_b) for a, b in zip(g, h))
         assert agree >= 24, f"only {agree}/32 tokens agree with full recompute at ratio 1.0"
+
+
+@pytest.mark.parametrize("use_acache", [True, False])
+def test_hip_graph_replay_of_refinement_steps_gives_the_same_tokens(device, use_acache):
+    """The captured refinement forward is replayed for every step of a block, with the engine's eager work (token
+    transfer, scheduling, the next block's refresh) between replays; every run must commit exactly the tokens of the
+    eager loop, and the graph must be re-captured when the attention metadata changes."""
+    cfg, model = _model(device, seed=3)
+    with torch.no_grad():
+        model.model.transformer["ff_out"].weight[63].zero_()
+    affix = list(range(20, 30))
+
+    def make(i):
+        return Sequence([2 + i] + affix + [40 + i, 41 + i], gen_length=16, block_length=8, cache_block_size=8,
+                        mask_id=63, prompt_affix_start=1, prompt_affix_end=11)
+
+    def run(graph):
+        serve = _serve(cfg, recompute_batch_size=2, max_num_seqs=0, gen_length=16, block_length=8,
+                       num_kvcache_blocks=48, threshold=0.9, anchor_ratio=0.5, enable_acache=use_acache,
+                       decode_hip_graph=graph)
+        runner = ModelRunner(model, serve)
+        seqs = [make(i) for i in range(3)]
+        out, nfe = (runner.generate_with_acache if use_acache else runner.generate_with_dual_cache)(seqs)
+        return out, nfe, runner.last_timing
+
+    eager, nfe_eager, _ = run(False)
+    for _ in range(2):   # twice: the second run captures without the eager warm-up forward
+        replayed, nfe_graph, timing = run(True)
+        assert replayed == eager and nfe_graph == nfe_eager
+        assert all(63 not in g for g in replayed)
