@@ -90,7 +90,42 @@ def cpu_relocation_baseline(torch, wl, budget_s=20.0):
                 sample=f"1 of {wl['layers']} layers of the same batch ({wl['T']} rows), median of {len(times)} runs after 2 warm-ups, {med * 1e3:.0f} ms each")
 
 
-def attention_bench(torch, device, ops, steps, warmup):
+def cpu_attention_baseline(torch, q, kc, vc, w, budget_s=15.0):
+    """Reference-style torch CPU path for the attention call: per request, gather K/V through the slot map and run
+    ``F.scaled_dot_product_attention`` over all heads (the formulation of nano-vdllm/model_runner.py:385-399), bf16
+    inputs up-cast to fp32.  Timed on a bounded sample of the 16 requests."""
+    import torch.nn.functional as F
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    H, D = q.shape[1], q.shape[2]
+    qc, kf, vf = q.cpu(), kc.cpu().view(-1, kc.shape[-2], D), vc.cpu().view(-1, vc.shape[-2], D)
+    cu_q, cu_k, slots = w["cu_q"].tolist(), w["cu_k"].tolist(), w["slot_map"].long()
+    sample = list(range(min(4, len(w["q_lens"]))))
+
+    def run():
+        for b in sample:
+            sl = slots[cu_k[b]:cu_k[b + 1]]
+            qb = qc[cu_q[b]:cu_q[b + 1]].float().transpose(0, 1)
+            kb = kf[sl].float().transpose(0, 1)
+            vb = vf[sl].float().transpose(0, 1)
+            F.scaled_dot_product_attention(qb, kb, vb).transpose(0, 1).to(torch.bfloat16)
+
+    times, t_begin = [], time.perf_counter()
+    for i in range(7):
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        if i >= 2:
+            times.append(dt)
+        if time.perf_counter() - t_begin > budget_s and times:
+            break
+    med = statistics.median(times)
+    flops = 4 * H * D * sum(w["q_lens"][b] * w["kv_lens"][b] for b in sample)
+    return dict(value=round(flops / med / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"{len(sample)} of {len(w['q_lens'])} requests of the same call, all 32 heads, median of {len(times)} runs after 2 warm-ups, {med * 1e3:.0f} ms each")
+
+
+def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
     """Anchor-recompute bidirectional varlen attention, one layer call: batch 16, 32 heads (MHA), D = 128, bf16."""
     from acache_amd.synthetic import attention_batch
 
@@ -116,7 +151,9 @@ def attention_bench(torch, device, ops, steps, warmup):
     kv_bytes = 2 * sum(w["kv_lens"]) * Hkv * D * 2
     qo_bytes = 2 * total_q * H * D * 2
     tflops = flops / (avg_ms * 1e-3) / 1e12
+    extra = {"cpu_baseline": cpu_attention_baseline(torch, q, kc, vc, w)} if cpu_baseline else {}
     return {
+        **extra,
         "metric": "anchor-recompute attn TFLOP/s", "value": round(tflops, 1), "unit": "TFLOP/s",
         "ms_per_call": round(avg_ms, 4),
         "config": {"workload": "configs[3]: batch 16, 32 heads (MHA), D 128, bf16, q = 20% anchors + 32 per request, "
@@ -411,7 +448,8 @@ def main():
     }
 
     if not args.no_attention:
-        result["attention"] = attention_bench(torch, device, ops, steps=max(args.steps, 20), warmup=args.warmup)
+        result["attention"] = attention_bench(torch, device, ops, steps=max(args.steps, 20), warmup=args.warmup,
+                                              cpu_baseline=not args.no_cpu_baseline)
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_relocation_baseline(torch, wl)
