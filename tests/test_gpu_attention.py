@@ -57,6 +57,28 @@ def test_ragged_lengths_plain_mode(device, H, Hkv, D):
     assert torch.all(got[cu_q[7]:cu_q[8]] == 0)
 
 
+@pytest.mark.parametrize("B", [64, 65, 150])
+def test_large_batches_on_both_sides_of_the_block_ordering_switch(device, B):
+    """Up to 64 requests the workgroups walk the requests longest first; above that in batch order.  Many requests
+    share a key count (ties in the ordering), some have no queries and some no keys."""
+    g = torch.Generator().manual_seed(B)
+    H, Hkv, D, S = 8, 8, 128, 2048
+    q_lens = torch.randint(0, 40, (B,), generator=g).tolist()
+    kv_lens = (torch.randint(0, 5, (B,), generator=g) * 48).tolist()     # 0, 48, ..., 192: plenty of ties
+    q_lens[3], kv_lens[5] = 0, 0
+    q = (torch.randn(sum(q_lens), H, D, generator=g) / D ** 0.25).to(torch.bfloat16)
+    kc = (torch.randn(S, Hkv, D, generator=g) / D ** 0.25).to(torch.bfloat16)
+    vc = torch.randn(S, Hkv, D, generator=g).to(torch.bfloat16)
+    slots = torch.cat([torch.randperm(S, generator=g)[:n] for n in kv_lens]).to(torch.int32)
+    cu_q = torch.tensor([0] + torch.tensor(q_lens).cumsum(0).tolist(), dtype=torch.int32)
+    cu_k = torch.tensor([0] + torch.tensor(kv_lens).cumsum(0).tolist(), dtype=torch.int32)
+    want = O.acache_attention(q, kc, vc, cu_q, cu_k, slots)
+    got = ops.acache_attention(q.to(device), kc.view(S // 16, 16, Hkv, D).to(device),
+                               vc.view(S // 16, 16, Hkv, D).to(device), cu_q.to(device), cu_k.to(device),
+                               slots.to(device))
+    _close(got, want)
+
+
 def test_invariants_on_device(device):
     torch.manual_seed(2)
     H, Hkv, D, S = 8, 2, 128, 2048
