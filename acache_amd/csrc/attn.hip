@@ -209,15 +209,13 @@ __device__ __forceinline__ void lds_dma16(const char *src, char *lds_dst) {
 //          has to stay within 2^8 of the true running maximum: probabilities up to 256 are
 //          harmless in fp32/bf16 and the final division by the running sum cancels the reference.
 //          The rescale of O (32 multiplies per lane and query tile) therefore runs only when some
-//          query's maximum jumped by more than 8 — one wave-uniform test for all query tiles,
-//          rarely true after the first tile.
+//          query's maximum jumped by more than 8 — one wave-uniform test per tile of 16 queries,
+//          rarely true after the first key tile.
 //   MASKED keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
 template <int NQ16, int NT, int DT, bool MASKED>
 __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], float (&m_run)[NQ16],
                                                   f32x4 (&l_acc)[NQ16], f32x4 (&o_acc)[NQ16][DT],
                                                   float c, int n_valid, int lg) {
-  float mxc[NQ16];
-  bool jump = false;
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
     if (MASKED) {
@@ -234,13 +232,11 @@ __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], floa
       for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
-    mxc[qt] = mx * c;
-    jump |= mxc[qt] > m_run[qt] + 8.0f;
-  }
-  if (__builtin_amdgcn_ballot_w64(jump) != 0) {
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt) {
-      const float m_new = fmaxf(m_run[qt], mxc[qt]);
+    const float mxc = mx * c;
+    // decided per tile of 16 queries, so a query row's arithmetic does not depend on which other rows share
+    // its wave (workgroups may give a wave one or two such tiles)
+    if (__builtin_amdgcn_ballot_w64(mxc > m_run[qt] + 8.0f) != 0) {
+      const float m_new = fmaxf(m_run[qt], mxc);
       const float m_use = m_new == -INFINITY ? 0.0f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
       l_acc[qt] *= alpha;
@@ -566,12 +562,14 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
 // 4*j + i/4, j = 0..3.  With lane l pointing at V[row0 + l/4][d0 + 4*(l%4)] lane i
 // gets V[row0 + 0..3][d0 + i]: four keys of one column, i.e. half of an MFMA
 // A-operand of V^T.
+// One query tile of one (request, head): the four waves take WQ = 16 * NQ16 query rows each, starting at
+// row q_tile0 of the request, and stream the request's K/V through the LDS ring.
 template <int DTYPE, int D, int NQ16, int MODE>
-__global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
-  static_assert(MODE != MODE_KEY_SIDE, "key-side rotation needs the register-staged kernel");
+__device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0, char *lds_v0, char *lds_k1,
+                                              char *lds_v1, int b, int q_begin, int q_len, int q_tile0, int head,
+                                              int kvh) {
   constexpr int BN = 64;
   constexpr int WQ = 16 * NQ16;
-  constexpr int BM = 4 * WQ;
   constexpr int KS = D / 32;
   constexpr int NT = BN / 16;
   constexpr int DT = D / 16;
@@ -585,58 +583,18 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
   constexpr int TILE_BYTES = BN * ROW_BYTES;
   using M = Mma<DTYPE>;
   typedef short s16x4 __attribute__((ext_vector_type(4)));
-
-  __shared__ __attribute__((aligned(16))) char lds_k0[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char lds_v0[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char lds_k1[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char lds_v1[TILE_BYTES];
-
-  // Block -> (query tile, head).  Consecutive block indices go to different XCDs (index mod 8), each
-  // with its own L2, so every XCD is given a contiguous range of KV heads: all query tiles that
-  // read a head's K/V find it in the same L2.  When the KV heads divide evenly among the XCDs,
-  // an XCD walks the query tiles in the outer loop (longest request first, see
-  // locate_query_tile_lpt) and its heads in the inner one; otherwise heads are outermost.
-  const int per_xcd = gridDim.x >> 3;
-  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
-  const int group = p.H / p.H_kv;
-  int tile, kvh, hg;
-  if (p.H_kv % 8 == 0) {
-    const int heads_per_xcd = (p.H_kv >> 3) * group;
-    tile = idx / heads_per_xcd;
-    if (tile >= p.num_tiles) return;
-    const int r = idx - tile * heads_per_xcd;
-    kvh = xcd * (p.H_kv >> 3) + r / group;
-    hg = r % group;
-  } else {
-    const int w = xcd * per_xcd + idx;
-    if (w >= p.num_tiles * p.H) return;
-    hg = w % group;
-    tile = (w / group) % p.num_tiles;
-    kvh = w / (group * p.num_tiles);
-  }
-  const int head = kvh * group + hg;
-  int b = 0, q_begin = 0, q_len = 0;
-  {
-    int tile_in_request = 0;
-    const bool found = p.B <= 64 ? locate_query_tile_lpt(p.cu_q, p.cu_k, p.B, BM, tile, b, q_begin, q_len, tile_in_request)
-                                 : locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request);
-    if (!found) return;
-    tile = tile_in_request;
-  }
-
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, lg = lane >> 4;
   const int kv_begin = p.cu_k[b];
   const int kv_len = p.cu_k[b + 1] - kv_begin;
-  const int q_tile0 = tile * BM;
   const int q_wave0 = q_tile0 + wave * WQ;
   int nq_valid = (q_len - q_wave0 + 15) / 16;
   nq_valid = nq_valid < 0 ? 0 : (nq_valid > NQ16 ? NQ16 : nq_valid);
   char *out_base = p.out + (int64_t)q_begin * p.o_token_bytes + (int64_t)head * p.o_head_bytes;
 
   if (kv_len <= 0) {
-    for (int r = tid / CH; r < BM; r += 256 / CH) {
+    for (int r = tid / CH; r < 4 * WQ; r += 256 / CH) {
       const int qr = q_tile0 + r;
       if (qr < q_len) store16(out_base + (int64_t)qr * p.o_token_bytes + (tid % CH) * 16, vec16{{0, 0, 0, 0}});
     }
@@ -946,6 +904,60 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
       }
     }
   }
+}
+
+template <int DTYPE, int D, int NQ16, int MODE>
+__global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
+  static_assert(MODE != MODE_KEY_SIDE, "key-side rotation needs the register-staged kernel");
+  constexpr int BM = 64 * NQ16;               // query rows per tile
+  constexpr int TILE_BYTES = 64 * D * 2;
+
+  __shared__ __attribute__((aligned(16))) char lds_k0[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char lds_v0[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char lds_k1[TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char lds_v1[TILE_BYTES];
+
+  // Block -> (query tile, head).  Consecutive block indices go to different XCDs (index mod 8), each
+  // with its own L2, so every XCD is given a contiguous range of KV heads: all query tiles that
+  // read a head's K/V find it in the same L2.  When the KV heads divide evenly among the XCDs,
+  // an XCD walks the query tiles in the outer loop (longest request first, see
+  // locate_query_tile_lpt) and its heads in the inner one; otherwise heads are outermost.
+  const int per_xcd = gridDim.x >> 3;
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int group = p.H / p.H_kv;
+  int tile, kvh, hg;
+  if (p.H_kv % 8 == 0) {
+    const int heads_per_xcd = (p.H_kv >> 3) * group;
+    tile = idx / heads_per_xcd;
+    if (tile >= p.num_tiles) return;
+    const int r = idx - tile * heads_per_xcd;
+    kvh = xcd * (p.H_kv >> 3) + r / group;
+    hg = r % group;
+  } else {
+    const int w = xcd * per_xcd + idx;
+    if (w >= p.num_tiles * p.H) return;
+    hg = w % group;
+    tile = (w / group) % p.num_tiles;
+    kvh = w / (group * p.num_tiles);
+  }
+  const int head = kvh * group + hg;
+  int b = 0, q_begin = 0, q_len = 0;
+  {
+    int tile_in_request = 0;
+    const bool found = p.B <= 64 ? locate_query_tile_lpt(p.cu_q, p.cu_k, p.B, BM, tile, b, q_begin, q_len, tile_in_request)
+                                 : locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request);
+    if (!found) return;
+    tile = tile_in_request;
+  }
+
+  // The last query tile of a request may hold few rows.  With at most half a tile left the four waves take
+  // 16 rows each instead of 32: the workgroup streams the same K/V but with half the matrix and softmax work per
+  // wave, and finishes in about two thirds of the time.
+  const int q_tile0 = tile * BM;
+  if (NQ16 == 2 && q_len - q_tile0 <= BM / 2)
+    attn_dma_tile<DTYPE, D, 1, MODE>(p, lds_k0, lds_v0, lds_k1, lds_v1, b, q_begin, q_len, q_tile0, head, kvh);
+  else
+    attn_dma_tile<DTYPE, D, NQ16, MODE>(p, lds_k0, lds_v0, lds_k1, lds_v1, b, q_begin, q_len, q_tile0, head, kvh);
 }
 
 template <int DTYPE, int D, int NQ16>
