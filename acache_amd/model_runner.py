@@ -425,36 +425,29 @@ class ModelRunner:
             self._add_timing_count(timing, "anchor_selection_kv_tokens", sum(len(s) for s in active_seqs))
             self._finish_timing(timing, "anchor_selection_prepare", start)
 
-            affix_slots = torch.arange(affix_len, dtype=torch.int32, device=self.device)
             uses_rope = bool(getattr(self.config.hf_config, "rope", True))
+            # one kernel pair per layer for the whole batch: softmax over the affix keys of every [MASK] query,
+            # column sums over queries and heads added to `importance` (the reference loops over requests here)
+            probe_rows = torch.cat(mask_positions).to(torch.int32)
+            counts = [int(rows.numel()) for rows in mask_positions]
+            probe_cu = self._to_device(np.concatenate([[0], np.cumsum(counts)]), torch.int32)
+            shifts = [seq.affix_start if uses_rope else 0 for seq in active_seqs]
+            probe_shifts = probe_cos = probe_sin = None
+            if any(shifts):
+                probe_shifts = self._to_device(shifts, torch.int32)
+                probe_sin, probe_cos = blocks[0].rotary_emb.get_rotary_embedding(
+                    max(self._affix_relocation_max_position, max(shifts) + 1), self.device)
+            probe_scratch = torch.empty(max(16, 8 * int(probe_rows.numel()) * blocks[0].attn.num_heads),
+                                        dtype=torch.uint8, device=self.device)
 
             def make_probe(layer_idx, block):
                 def probe(attention, q):
-                    q_heads = q.reshape(-1, attention.num_heads, attention.head_dim)
-                    rotated = {}
-                    for b, seq in enumerate(active_seqs):
-                        rows = mask_positions[b]
-                        if rows.numel() == 0:
-                            continue
-                        shift = seq.affix_start if uses_rope else 0
-                        if shift not in rotated:
-                            if shift == 0:
-                                rotated[shift] = self._shared_affix_k(layer_idx)
-                            else:  # cached keys sit at positions 0..A-1: move them to affix_start..
-                                sin, cos = block.rotary_emb.get_rotary_embedding(
-                                    max(self._affix_relocation_max_position, shift + 1), self.device)
-                                cache_l = attention.k_cache.view(1, -1, attention.num_kv_heads, attention.head_dim)
-                                deltas = torch.full((affix_len,), shift, dtype=torch.int32, device=self.device)
-                                rotated[shift] = ops.relocate_rope_gather(
-                                    cache_l, attention.v_cache.view_as(cache_l), affix_slots, deltas, cos, sin)[0][0]
-                        affix_k = rotated[shift].permute(1, 0, 2)
-                        groups = attention.num_heads // affix_k.shape[0]
-                        if groups > 1:
-                            affix_k = affix_k.repeat_interleave(groups, dim=0)
-                        seq_q = q_heads.index_select(0, rows).permute(1, 0, 2)
-                        scale = attention.scale if attention.scale is not None else attention.head_dim ** -0.5
-                        weights = torch.softmax(torch.matmul(seq_q, affix_k.transpose(-2, -1)) * scale, dim=-1)
-                        importance[b].add_(weights.sum(dim=-2).sum(dim=-2).float())
+                    if probe_rows.numel() == 0:
+                        return
+                    ops.affix_importance(
+                        importance, q.reshape(-1, attention.num_heads, attention.head_dim), attention.k_cache,
+                        probe_rows, probe_cu, affix_len, max(counts), attention.scale, probe_shifts, probe_cos,
+                        probe_sin, affix_slot0=0, workspace=probe_scratch)
                 return probe
 
             for layer_idx, block in enumerate(blocks):

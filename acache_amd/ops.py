@@ -266,6 +266,60 @@ def argmax_confidence(logits: torch.Tensor, picks: torch.Tensor | None = None):
     return token.view(logits.shape[:-1]), conf.view(logits.shape[:-1])
 
 
+def affix_importance(
+    importance: torch.Tensor,
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    mask_rows: torch.Tensor,
+    cu_mask: torch.Tensor,
+    affix_len: int,
+    max_mask_rows: int,
+    softmax_scale: float | None = None,
+    affix_shifts: torch.Tensor | None = None,
+    rope_cos: torch.Tensor | None = None,
+    rope_sin: torch.Tensor | None = None,
+    affix_slot0: int = 0,
+    workspace: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """Add one layer's affix importance to ``importance`` (fp32 ``[B, >= affix_len]``).
+
+    For each request the [MASK] queries ``q[mask_rows[cu_mask[b]:cu_mask[b+1]]]`` attend to the cached affix keys
+    ``k_cache`` slots ``affix_slot0 .. + affix_len`` (re-rotated by ``affix_shifts[b]``); the softmax runs over the
+    affix keys only and its columns are summed over queries and heads (nano-vdllm/model_runner.py:730-773).
+    ``workspace``: optional uint8 scratch of ``affix_importance_workspace_bytes`` bytes, allocated here if absent.
+    """
+    Tq, H, D = q.shape
+    H_kv = k_cache.shape[-2]
+    kc = k_cache.view(-1, H_kv, D)
+    assert importance.dtype == torch.float32 and importance.dim() == 2 and importance.stride(1) == 1
+    assert q.is_cuda and q.dtype == kc.dtype and q.stride(-1) == 1 and kc.is_contiguous()
+    B = cu_mask.numel() - 1
+    assert importance.shape[0] >= B and importance.shape[1] >= affix_len
+    rows = _i32(mask_rows, "mask_rows")
+    cu = _i32(cu_mask, "cu_mask")
+    total = rows.numel()
+    relocate = affix_shifts is not None
+    if relocate and (rope_cos is None or rope_sin is None):
+        raise ValueError("Post-RoPE affix relocation requires shifts and RoPE tables.")
+    shifts = _i32(affix_shifts, "affix_shifts") if relocate else None
+    scale = softmax_scale if softmax_scale is not None else D ** -0.5
+    lib = _lib.load()
+    need = lib.acache_affix_importance_workspace_bytes(total, H)
+    if workspace is None:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    assert workspace.is_cuda and workspace.numel() * workspace.element_size() >= need
+    with torch.cuda.device(q.device):
+        rc = lib.acache_affix_importance(
+            _ptr(importance), _ptr(q), _ptr(kc), _ptr(rows), _ptr(cu), _ptr(shifts),
+            _ptr(rope_cos) if relocate else None, _ptr(rope_sin) if relocate else None,
+            rope_cos.shape[0] if relocate else 0, float(scale),
+            affix_len, affix_slot0, B, total, max_mask_rows, H, H_kv, D, _code(q), kc.shape[0],
+            importance.stride(0), q.stride(0), q.stride(1), kc.stride(0), kc.stride(1),
+            _ptr(workspace), workspace.numel() * workspace.element_size(), _stream(q))
+    _lib.check(rc, "affix_importance")
+    return importance
+
+
 def kv_scatter_layers(
     key: torch.Tensor,
     value: torch.Tensor,

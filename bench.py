@@ -259,6 +259,20 @@ def kernel_sweep(torch, device, ops, steps):
         sl = torch.randperm(kc.shape[0] * 256, device=device)[:n_tok].to(torch.int32)
         row("rope_scatter_kernel", timed(lambda: ops.rope_qk_scatter(q, k, v, pos, cos, sin, kc, vc, sl)),
             n_tok * H * D * 2 * (3 + 4), f"{what}, 32 heads x 128, bf16 (q, k, v read; q, k, K-slot, V-slot written)")
+    # anchor-selection probe of one layer: 16 requests x 256 [MASK] queries against 1 000 shared affix keys
+    B, M, A = 16, 256, 1000
+    qp = (torch.randn(B * M, H, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    kp = (torch.randn(1024, H, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    rows_p = torch.arange(B * M, dtype=torch.int32, device=device)
+    cu_p = torch.arange(0, (B + 1) * M, M, dtype=torch.int32, device=device)
+    sh_p = torch.randint(1, 256, (B,), generator=gen, device=device).to(torch.int32)
+    imp = torch.zeros(B, A, dtype=torch.float32, device=device)
+    ws = torch.empty(8 * B * M * H, dtype=torch.uint8, device=device)
+    us = timed(lambda: ops.affix_importance(imp, qp, kp, rows_p, cu_p, A, M, None, sh_p, cos, sin, 0, ws))
+    flops = 2 * 2 * B * M * A * H * D   # the scores are computed twice (row statistics, then column sums)
+    out.append({"kernel": "importance_stats_kernel + importance_colsum_kernel", "us": round(us, 1),
+                "TFLOPs": round(flops / us / 1e6, 1), "flops": flops,
+                "workload": "one layer: 16 requests x 256 mask queries x 1 000 affix keys, 32 heads x 128, bf16, key-side re-rotation"})
     logits = torch.randn(512, 126464, generator=gen, device=device).to(torch.bfloat16)
     row("confidence_kernel", timed(lambda: ops.argmax_confidence(logits)), 512 * 126464 * 2,
         "512 rows x 126 464 logits, bf16")

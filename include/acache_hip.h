@@ -8,7 +8,8 @@
  *
  * Conventions shared by every entry point
  *   - all data pointers are DEVICE pointers owned by the caller; nothing is
- *     allocated, freed or retained by the library;
+ *     allocated, freed or retained by the library (the one entry point that needs
+ *     scratch memory, acache_affix_importance, takes it as a workspace argument);
  *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
  *     default stream) and the call returns without synchronising;
  *   - return value: 0 = enqueued; < 0 = argument error (ACACHE_E_*), nothing was
@@ -159,6 +160,39 @@ int acache_rope_qk_scatter(
     int64_t N, int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
     int64_t q_token_stride, int64_t k_token_stride, int64_t v_token_stride,
     void *stream);
+
+/*
+ * Affix importance for anchor selection: attention of each request's [MASK] queries
+ * to the cached affix keys, soft-maxed over the affix keys only, summed over the
+ * mask queries and the heads of one layer and ADDED to importance[b, :].
+ *
+ *   for b < B, r in mask_rows[cu_mask[b] .. cu_mask[b+1]), h < H:
+ *     w[a] = softmax_a( q[r, h] . rot(k_cache[affix_slot0 + a, h / (H/H_kv)], affix_shifts[b]) * scale ), a < affix_len
+ *     importance[b, a] += w[a]
+ *   rot as in acache_relocate_rope_gather (rounded to `dtype`); fp32 scores and softmax.
+ *
+ * Replaces the per-request loop of the patched attention forward in
+ * _compute_anchor_positions_batch (nano-vdllm/model_runner.py:730-773: rotary
+ * re-application on the cached affix keys, matmul, softmax, two sums, add_), once
+ * per layer; call it for every layer on the same importance buffer, then
+ * acache_topk_anchors.  The reference evaluates matmul and softmax in the model
+ * dtype; here they are fp32.  Deterministic: no atomics, fixed summation order.
+ *
+ * mask_rows are row indices into q ([Tq, H, D] with the given strides).  workspace:
+ * device scratch of at least acache_affix_importance_workspace_bytes(total_mask_rows, H)
+ * bytes (row statistics between the two launches), 16-byte aligned, owned by the
+ * caller.  max_mask_rows: an upper bound on the mask rows of one request.
+ */
+int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_rows, int32_t H);
+int acache_affix_importance(
+    float *importance, const void *q, const void *k_cache,
+    const int32_t *mask_rows, const int32_t *cu_mask, const int32_t *affix_shifts,
+    const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows,
+    int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int64_t importance_stride, int64_t q_token_stride, int64_t q_head_stride,
+    int64_t kv_slot_stride, int64_t kv_head_stride,
+    void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
  * Per-request top-k anchor selection over ragged fp32 influence scores.

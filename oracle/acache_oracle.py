@@ -99,6 +99,38 @@ def argmax_confidence(logits, picks=None):
     return x0.view(logits.shape[:-1]), conf.view(logits.shape[:-1])
 
 
+def affix_importance(q, k_cache, mask_rows, cu_mask, affix_len, scale=None, affix_shifts=None, cos=None, sin=None,
+                     affix_slot0=0):
+    """One layer's affix importance ``[B, affix_len]`` fp32 (nano-vdllm/model_runner.py:730-773).
+
+    Per request: the cached affix keys (slots ``affix_slot0 ..``, cached at positions ``0 .. A-1``) are re-rotated
+    to start at ``affix_shifts[b]`` (rounded to the cache dtype, like ``block.rotary_emb`` there), the [MASK]
+    queries are scored against them, the softmax runs over the affix keys only, and the weights are summed over
+    queries and heads.  The reference evaluates ``matmul`` / ``softmax`` in the model dtype; this restatement uses
+    fp32 for both, which is what the bound "within tolerance" is stated against.
+    """
+    H, D = q.shape[1], q.shape[2]
+    flat = _flat(k_cache)
+    H_kv = flat.shape[1]
+    scale = D ** -0.5 if scale is None else scale
+    B = len(cu_mask) - 1
+    out = torch.zeros(B, affix_len, dtype=torch.float32)
+    keys = flat[affix_slot0:affix_slot0 + affix_len]
+    for b in range(B):
+        rows = mask_rows[int(cu_mask[b]):int(cu_mask[b + 1])].long()
+        if rows.numel() == 0 or affix_len == 0:
+            continue
+        k = keys
+        shift = int(affix_shifts[b]) if affix_shifts is not None else 0
+        if shift:
+            k = rotate(keys, torch.full((affix_len,), shift, dtype=torch.int32), cos, sin)
+        kh = k.float().permute(1, 0, 2).repeat_interleave(H // H_kv, dim=0)          # [H, A, D]
+        qh = q[rows].float().permute(1, 0, 2)                                           # [H, M, D]
+        w = torch.softmax(torch.matmul(qh, kh.transpose(-2, -1)) * scale, dim=-1)       # [H, M, A]
+        out[b] = w.sum(dim=(0, 1))
+    return out
+
+
 def rotate(x: torch.Tensor, delta: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
     """Rotate rows ``x[t]`` (``[T, H, D]``) by signed per-row position shifts ``delta[t]``.
 

@@ -365,3 +365,32 @@ def test_get_transfer_index_closed_form():
     x0, t = O.get_transfer_index(logits, torch.tensor([[False, True, True]]), x, threshold=0.9)
     assert x0.tolist() == [[9, 0, 0]]
     assert t.tolist() == [[False, False, True]]      # nothing reaches 0.9: force the most confident masked row
+
+
+# ------------------------------------------------------------------ affix importance (model_runner.py:730-773)
+def test_affix_importance_closed_forms_and_brute_force():
+    g = torch.Generator().manual_seed(11)
+    H, Hkv, D, A, S = 4, 2, 64, 9, 16
+    cos, sin = O.rope_table(64, D, 1e4)
+    kc = torch.randn(S, Hkv, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(12, H, D, generator=g).to(torch.bfloat16)
+    mask_rows = torch.tensor([1, 4, 5, 7, 8, 9, 10], dtype=torch.int32)
+    cu = torch.tensor([0, 3, 3, 7], dtype=torch.int32)            # request 1 has no [MASK] query
+    shifts = torch.tensor([0, 5, 11], dtype=torch.int32)
+    imp = O.affix_importance(q, kc, mask_rows, cu, A, affix_shifts=shifts, cos=cos, sin=sin, affix_slot0=2)
+    assert imp.shape == (3, A)
+    # every softmax row sums to one: the total is (mask rows) x (heads)
+    assert torch.allclose(imp.sum(1), torch.tensor([3.0 * H, 0.0, 4.0 * H]), atol=1e-4)
+    # brute force of the definition, request 2 (shift 11)
+    kr = O.rotate(kc[2:2 + A], torch.full((A,), 11, dtype=torch.int32), cos, sin).float()
+    want = torch.zeros(A)
+    for r in mask_rows[3:7].tolist():
+        for h in range(H):
+            s = torch.tensor([float(q[r, h].float() @ kr[a, h // 2]) for a in range(A)]) * D ** -0.5
+            want += torch.softmax(s, 0)
+    assert torch.allclose(imp[2], want, atol=1e-4)
+    # identical keys: every affix token gets the same share
+    same = kc.clone()
+    same[:] = kc[0]
+    u = O.affix_importance(q, same, mask_rows, cu, A)
+    assert torch.allclose(u[0], torch.full((A,), 3.0 * H / A), atol=1e-5)
