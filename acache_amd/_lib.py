@@ -33,7 +33,7 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         c_int32, c_int64, c_int32, c_int32, c_int32, c_int32, c_int64,
         c_int64, c_int64, c_int64, c_void_p]),
-    "acache_affix_importance_workspace_bytes": (c_int64, [c_int64, c_int32]),
+    "acache_affix_importance_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32]),
     "acache_affix_importance": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float,
         c_int32, c_int64, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,

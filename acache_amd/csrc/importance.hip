@@ -5,15 +5,18 @@
 //   w[r, h, a]       = softmax_a( q[r, h] . rot(K[a, kv(h)], shift_b) * scale )     a in [0, A)
 //   importance[b, a] += sum_{r in mask rows of b} sum_h w[r, h, a]
 //
-// Two launches, no atomics, so the result does not depend on scheduling:
-//   1. importance_stats_kernel: one wave per (request, head, 16 mask rows) walks the affix keys and
+// Three launches (four with relocation: the cached keys of every request are first re-rotated once into the
+// workspace), no atomics, so the result does not depend on scheduling:
+//   1. importance_stats_kernel: one wave per (request, head, 64 mask rows) walks the affix keys and
 //      leaves the row maximum and the row sum of exp (log2 domain) in the workspace;
-//   2. importance_colsum_kernel: one wave per (request, 32 affix keys) walks the heads and the mask
-//      rows, recomputes the scores, normalises them with the stored row statistics and accumulates
-//      the column sums in registers; it is the only writer of its 32 entries of importance[b, :].
+//   2. importance_colsum_kernel: one wave per (request, head, 64 affix keys) keeps its keys in
+//      registers, walks the request's mask rows, recomputes the scores, normalises them with the
+//      stored row statistics and sums the columns; it is the only writer of its 64 entries of the
+//      per-head partial sums in the workspace;
+//   3. importance_reduce_kernel adds the per-head partial sums, in head order, to importance[b, :].
 // Scores come from the matrix core (S^T = K Q^T, keys as rows, one query column per lane).  K and Q
-// fragments are loaded straight from global memory in operand layout (16 bytes per lane) and the
-// cached keys are re-rotated in registers; nothing goes through LDS and there is no barrier.
+// fragments are loaded straight from global memory in operand layout (16 bytes per lane); nothing goes
+// through LDS and there is no barrier.
 #include "common.h"
 #include "mma.h"
 
@@ -29,6 +32,9 @@ struct ImportanceParams {
   const float *cos_tab;
   const float *sin_tab;
   float2 *stats;
+  float *partial;
+  char *k_rot;            // [B, A, H_kv, D] re-rotated affix keys (NULL: read the cache directly)
+  int64_t k_rot_bytes;    // per request
   int64_t imp_stride;
   int64_t q_token_bytes, q_head_bytes;
   int64_t kv_slot_bytes, kv_head_bytes;
@@ -57,106 +63,181 @@ __device__ __forceinline__ void load_rows(vec16 (&f)[D / 32], const char *row_pt
   }
 }
 
+// Re-rotate the cached affix keys once per request: k_rot[b, a, h, :] = rot(K[affix_slot0 + a, h, :], shift_b).
+// One row of D elements per LPR lanes, the rotate-half partner in the same lane; fp32 products and sum rounded
+// separately, one rounding to the cache type (the arithmetic of the relocation kernel).
+template <int DTYPE, int D>
+__global__ __launch_bounds__(256) void importance_rotate_kernel(ImportanceParams p) {
+#pragma clang fp contract(off)
+  using E = Elem<DTYPE>;
+  constexpr int VEC = E::kPerVec;
+  constexpr int HALF_BYTES = D * E::kBytes / 2;
+  constexpr int LPR = HALF_BYTES / 16;
+  constexpr int RPB = 256 / LPR;
+  const int b = blockIdx.y;
+  const int lane = threadIdx.x % LPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+  if (row >= (int64_t)p.A * p.H_kv) return;
+  const int64_t a = row / p.H_kv;
+  const int head = (int)(row - a * p.H_kv);
+  int shift = p.shifts[b];
+  if (shift < 0 || shift >= p.rope_rows) shift = 0;
+  const char *src = p.k_cache + (p.affix_slot0 + a) * p.kv_slot_bytes + (int64_t)head * p.kv_head_bytes + lane * 16;
+  char *dst = p.k_rot + (int64_t)b * p.k_rot_bytes + row * (2 * HALF_BYTES) + lane * 16;
+  vec16 lo = load16(src), hi = load16(src + HALF_BYTES);
+  if (shift != 0) {
+    const float *cr = p.cos_tab + (int64_t)shift * D + lane * VEC;
+    const float *sr = p.sin_tab + (int64_t)shift * D + lane * VEC;
+    float x[VEC], y[VEC], xa[VEC], ya[VEC];
+    E::unpack(lo, x);
+    E::unpack(hi, y);
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) {
+      xa[j] = x[j] * cr[j] + (-y[j]) * sr[j];
+      ya[j] = y[j] * cr[D / 2 + j] + x[j] * sr[D / 2 + j];
+    }
+    lo = E::pack(xa);
+    hi = E::pack(ya);
+  }
+  store16(dst, lo);
+  store16(dst + HALF_BYTES, hi);
+}
+
+constexpr int kKeysPerStep = 64;  // keys a wave scores per loop step (four independent 16-key tiles in flight)
+
+constexpr int kRowTilesPerWave = 4;  // 16-row tiles of mask queries a stats wave owns (keys are loaded once for all)
+
 template <int DTYPE, int D>
 __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams p) {
   constexpr int KS = D / 32;
+  constexpr int NQ = kRowTilesPerWave;
   using M = Mma<DTYPE>;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
-  const int b = blockIdx.x / p.max_row_tiles, rt = blockIdx.x % p.max_row_tiles;
+  const int groups = (p.max_row_tiles + NQ - 1) / NQ;
+  const int b = blockIdx.x / groups, rg = blockIdx.x % groups;
   const int h = blockIdx.y * 4 + wave;
   const int m0 = p.cu_mask[b];
   const int n_rows = p.cu_mask[b + 1] - m0;
-  if (h >= p.H || rt * 16 >= n_rows) return;  // no barrier in this kernel: waves may leave early
+  const int row0 = rg * NQ * 16;
+  if (h >= p.H || row0 >= n_rows) return;  // no barrier in this kernel: waves may leave early
   const int kvh = h / (p.H / p.H_kv);
 
-  const int r = rt * 16 + li;
-  vec16 qf[KS];
-  load_rows<DTYPE, D>(qf, r < n_rows ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
-                                     : nullptr, lg, nullptr, nullptr);
-  int shift = p.shifts ? p.shifts[b] : 0;
-  if (shift < 0 || shift >= p.rope_rows) shift = 0;
-  const float *cr = shift ? p.cos_tab + (int64_t)shift * D : nullptr;
-  const float *sr = shift ? p.sin_tab + (int64_t)shift * D : nullptr;
-  const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
+  vec16 qf[NQ][KS];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    const int r = row0 + 16 * qt + li;
+    load_rows<DTYPE, D>(qf[qt], r < n_rows ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
+                                           : nullptr, lg, nullptr, nullptr);
+  }
+  const int64_t slot_bytes = p.k_rot ? (int64_t)p.H_kv * D * 2 : p.kv_slot_bytes;
+  const char *k_base = p.k_rot ? p.k_rot + (int64_t)b * p.k_rot_bytes + (int64_t)kvh * D * 2
+                               : p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
   const float c = p.scale_log2e;
 
-  float m_run = -INFINITY, l_run = 0.0f;  // per query column (lane li); l is this lane group's share
-  for (int a0 = 0; a0 < p.A; a0 += 16) {
-    vec16 kf[KS];
-    load_rows<DTYPE, D>(kf, a0 + li < p.A ? k_base + (int64_t)(a0 + li) * p.kv_slot_bytes : nullptr, lg, cr, sr);
-    f32x4 s = {0, 0, 0, 0};
+  float m_run[NQ], l_run[NQ];  // per query column (lane li); l is this lane group's share
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) s = M::run(kf[ks], qf[ks], s);
-    float mx = -INFINITY;
+  for (int qt = 0; qt < NQ; ++qt) { m_run[qt] = -INFINITY; l_run[qt] = 0.0f; }
+  for (int a0 = 0; a0 < p.A; a0 += kKeysPerStep) {
+    vec16 kf[4][KS];  // 64 keys: rows a0 + 16*nt + li
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (a0 + 4 * lg + i >= p.A) s[i] = -INFINITY;
-      mx = fmaxf(mx, s[i]);
+    for (int nt = 0; nt < 4; ++nt) {
+      const int a = a0 + 16 * nt + li;
+      load_rows<DTYPE, D>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, nullptr, nullptr);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float m_new = fmaxf(m_run, mx * c);  // finite: every tile holds at least one existing key
-    float add = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(s[i] * c - m_new);
-    l_run = l_run * __builtin_amdgcn_exp2f(m_run - m_new) + add;
-    m_run = m_new;
+    for (int qt = 0; qt < NQ; ++qt) {
+      f32x4 s[4];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        s[nt] = f32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) s[nt] = M::run(kf[nt][ks], qf[qt][ks], s[nt]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (a0 + 16 * nt + 4 * lg + i >= p.A) s[nt][i] = -INFINITY;
+          mx = fmaxf(mx, s[nt][i]);
+        }
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run[qt], mx * c);  // finite: every step holds at least one existing key
+      float add = 0.0f;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(s[nt][i] * c - m_new);
+      l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + add;
+      m_run[qt] = m_new;
+    }
   }
-  l_run += __shfl_xor(l_run, 16);
-  l_run += __shfl_xor(l_run, 32);
-  if (lg == 0 && r < n_rows) p.stats[(int64_t)(m0 + r) * p.H + h] = make_float2(m_run, l_run);
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    float l = l_run[qt];
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    const int r = row0 + 16 * qt + li;
+    if (lg == 0 && r < n_rows) p.stats[(int64_t)(m0 + r) * p.H + h] = make_float2(m_run[qt], l);
+  }
 }
 
+// One wave per (request, head, 64 affix keys): the keys stay in registers, the request's mask rows stream by.
+// The wave is the only writer of partial[b, h, a0 .. a0 + 64).
 template <int DTYPE, int D>
 __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams p) {
   constexpr int KS = D / 32;
-  constexpr int NTW = 2;  // 16-key tiles per wave
   using M = Mma<DTYPE>;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
-  const int b = blockIdx.y;
-  const int a0 = (blockIdx.x * 4 + wave) * 16 * NTW;
+  const int b = blockIdx.z;
+  const int h = blockIdx.y * 4 + wave;
+  const int a0 = blockIdx.x * kKeysPerStep;
   const int m0 = p.cu_mask[b];
   const int n_rows = p.cu_mask[b + 1] - m0;
-  if (a0 >= p.A || n_rows <= 0) return;
-  int shift = p.shifts ? p.shifts[b] : 0;
-  if (shift < 0 || shift >= p.rope_rows) shift = 0;
-  const float *cr = shift ? p.cos_tab + (int64_t)shift * D : nullptr;
-  const float *sr = shift ? p.sin_tab + (int64_t)shift * D : nullptr;
+  if (h >= p.H) return;
   const float c = p.scale_log2e;
-  const int group = p.H / p.H_kv;
+  const int kvh = h / (p.H / p.H_kv);
+  const int64_t slot_bytes = p.k_rot ? (int64_t)p.H_kv * D * 2 : p.kv_slot_bytes;
+  const char *k_base = p.k_rot ? p.k_rot + (int64_t)b * p.k_rot_bytes + (int64_t)kvh * D * 2
+                               : p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
 
-  float col[NTW][4] = {};
-  for (int h = 0; h < p.H; ++h) {
-    const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)(h / group) * p.kv_head_bytes;
-    vec16 kf[NTW][KS];
+  vec16 kf[4][KS];
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt) {
-      const int a = a0 + 16 * nt + li;
-      load_rows<DTYPE, D>(kf[nt], a < p.A ? k_base + (int64_t)a * p.kv_slot_bytes : nullptr, lg, cr, sr);
+  for (int nt = 0; nt < 4; ++nt) {
+    const int a = a0 + 16 * nt + li;
+    load_rows<DTYPE, D>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, nullptr, nullptr);
+  }
+  float col[4][4] = {};
+  auto fetch = [&](int r0, vec16 (&qf)[KS], float2 &st) __attribute__((always_inline)) {
+    const int r = r0 + li;
+    const bool live = r < n_rows;
+    load_rows<DTYPE, D>(qf, live ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
+                                 : nullptr, lg, nullptr, nullptr);
+    st = live ? p.stats[(int64_t)(m0 + r) * p.H + h] : make_float2(0.0f, INFINITY);  // 1 / inf = 0: adds nothing
+  };
+  vec16 q_cur[KS], q_next[KS];
+  float2 st_cur, st_next;
+  if (n_rows > 0) fetch(0, q_cur, st_cur);
+  for (int r0 = 0; r0 < n_rows; r0 += 16) {
+    if (r0 + 16 < n_rows) fetch(r0 + 16, q_next, st_next);  // next row tile on its way while this one is scored
+    const float inv_l = 1.0f / st_cur.y;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      f32x4 s = {0, 0, 0, 0};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) s = M::run(kf[nt][ks], q_cur[ks], s);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(s[i] * c - st_cur.x) * inv_l;
     }
-    for (int r0 = 0; r0 < n_rows; r0 += 16) {
-      const int r = r0 + li;
-      const bool live = r < n_rows;
-      vec16 qf[KS];
-      load_rows<DTYPE, D>(qf, live ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
-                                   : nullptr, lg, nullptr, nullptr);
-      const float2 st = live ? p.stats[(int64_t)(m0 + r) * p.H + h] : make_float2(0.0f, 1.0f);
-      const float inv_l = live ? 1.0f / st.y : 0.0f;  // rows past the end add nothing
 #pragma unroll
-      for (int nt = 0; nt < NTW; ++nt) {
-        f32x4 s = {0, 0, 0, 0};
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s = M::run(kf[nt][ks], qf[ks], s);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(s[i] * c - st.x) * inv_l;
-      }
-    }
+    for (int ks = 0; ks < KS; ++ks) q_cur[ks] = q_next[ks];
+    st_cur = st_next;
   }
   // sum over the 16 query columns (lanes li) of every key row
+  float *dst = p.partial + ((int64_t)b * p.H + h) * p.A;
 #pragma unroll
-  for (int nt = 0; nt < NTW; ++nt)
+  for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float v = col[nt][i];
@@ -165,16 +246,40 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
       v += __shfl_xor(v, 4);
       v += __shfl_xor(v, 8);
       const int a = a0 + 16 * nt + 4 * lg + i;
-      if (li == 0 && a < p.A) p.importance[(int64_t)b * p.imp_stride + a] += v;
+      if (li == 0 && a < p.A) dst[a] = v;
     }
+}
+
+// importance[b, a] += sum over heads, in head order, of partial[b, h, a].
+__global__ __launch_bounds__(256) void importance_reduce_kernel(ImportanceParams p) {
+  const int a = blockIdx.x * 256 + threadIdx.x;
+  const int b = blockIdx.y;
+  if (a >= p.A) return;
+  const float *src = p.partial + (int64_t)b * p.H * p.A + a;
+  float acc = 0.0f;
+  for (int h = 0; h < p.H; ++h) acc += src[(int64_t)h * p.A];
+  p.importance[(int64_t)b * p.imp_stride + a] += acc;
 }
 
 }  // namespace acache
 
 using namespace acache;
 
-extern "C" int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_rows, int32_t H) {
-  return total_mask_rows < 0 || H < 0 ? 0 : total_mask_rows * H * (int64_t)sizeof(float2);
+static int64_t stats_bytes(int64_t total_mask_rows, int32_t H) {
+  return (total_mask_rows * H * (int64_t)sizeof(float2) + 15) / 16 * 16;
+}
+
+static int64_t partial_bytes(int32_t B, int32_t H, int32_t affix_len) {
+  return ((int64_t)B * H * affix_len * (int64_t)sizeof(float) + 15) / 16 * 16;
+}
+
+extern "C" int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_rows, int32_t B, int32_t H,
+                                                           int32_t H_kv, int32_t D, int32_t affix_len,
+                                                           int32_t relocated) {
+  if (total_mask_rows < 0 || B < 0 || H < 0 || H_kv < 0 || D < 0 || affix_len < 0) return 0;
+  if (relocated)  // one re-rotated copy of the affix keys per request (2-byte elements)
+    return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) + (int64_t)B * affix_len * H_kv * D * 2;
+  return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len);
 }
 
 extern "C" int acache_affix_importance(
@@ -199,9 +304,9 @@ extern "C" int acache_affix_importance(
     return fail(ACACHE_E_RANGE, "affix_importance: affix slots [%lld, %lld) outside %lld slots", (long long)affix_slot0,
                 (long long)(affix_slot0 + affix_len), (long long)num_slots);
   if (importance_stride < affix_len) return fail(ACACHE_E_SHAPE, "affix_importance: importance stride < affix_len");
-  if (workspace_bytes < acache_affix_importance_workspace_bytes(total_mask_rows, H))
+  if (workspace_bytes < acache_affix_importance_workspace_bytes(total_mask_rows, B, H, H_kv, D, affix_len, affix_shifts != nullptr))
     return fail(ACACHE_E_SHAPE, "affix_importance: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
-                (long long)acache_affix_importance_workspace_bytes(total_mask_rows, H));
+                (long long)acache_affix_importance_workspace_bytes(total_mask_rows, B, H, H_kv, D, affix_len, affix_shifts != nullptr));
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(workspace) || (rope_cos && !aligned16(rope_cos)) ||
       (rope_sin && !aligned16(rope_sin)) || (q_token_stride * 2) % 16 || (q_head_stride * 2) % 16 ||
       (kv_slot_stride * 2) % 16 || (kv_head_stride * 2) % 16)
@@ -210,6 +315,9 @@ extern "C" int acache_affix_importance(
   p.importance = importance; p.q = (const char *)q; p.k_cache = (const char *)k_cache;
   p.mask_rows = mask_rows; p.cu_mask = cu_mask; p.shifts = affix_shifts;
   p.cos_tab = rope_cos; p.sin_tab = rope_sin; p.stats = (float2 *)workspace;
+  p.partial = (float *)((char *)workspace + stats_bytes(total_mask_rows, H));
+  p.k_rot_bytes = (int64_t)affix_len * H_kv * D * 2;
+  p.k_rot = affix_shifts ? (char *)workspace + stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) : nullptr;
   p.imp_stride = importance_stride;
   p.q_token_bytes = q_token_stride * 2; p.q_head_bytes = q_head_stride * 2;
   p.kv_slot_bytes = kv_slot_stride * 2; p.kv_head_bytes = kv_head_stride * 2;
@@ -218,15 +326,27 @@ extern "C" int acache_affix_importance(
   p.A = affix_len; p.B = B; p.H = H; p.H_kv = H_kv; p.rope_rows = rope_rows;
   p.max_row_tiles = (max_mask_rows + 15) / 16;
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid1((unsigned)((int64_t)B * p.max_row_tiles), (unsigned)((H + 3) / 4));
-  const dim3 grid2((unsigned)((affix_len + 127) / 128), (unsigned)B);
+  const int rows_per_block = 256 / (D * 2 / 32);
+  const dim3 grid0((unsigned)(((int64_t)affix_len * H_kv + rows_per_block - 1) / rows_per_block), (unsigned)B);
+  const int row_groups = (p.max_row_tiles + kRowTilesPerWave - 1) / kRowTilesPerWave;
+  const dim3 grid1((unsigned)((int64_t)B * row_groups), (unsigned)((H + 3) / 4));
+  const dim3 grid2((unsigned)((affix_len + kKeysPerStep - 1) / kKeysPerStep), (unsigned)((H + 3) / 4), (unsigned)B);
+  const dim3 grid3((unsigned)((affix_len + 255) / 256), (unsigned)B);
 #define ACACHE_CASE(DT, DD)                                                                       \
   if (dtype == DT && D == DD) {                                                                   \
+    if (p.k_rot) {                                                                                \
+      hipLaunchKernelGGL((importance_rotate_kernel<DT, DD>), grid0, dim3(256), 0, s, p);          \
+      const int rc0 = launch_status("importance_rotate_kernel");                                  \
+      if (rc0) return rc0;                                                                        \
+    }                                                                                             \
     hipLaunchKernelGGL((importance_stats_kernel<DT, DD>), grid1, dim3(256), 0, s, p);             \
     const int rc = launch_status("importance_stats_kernel");                                      \
     if (rc) return rc;                                                                            \
     hipLaunchKernelGGL((importance_colsum_kernel<DT, DD>), grid2, dim3(256), 0, s, p);            \
-    return launch_status("importance_colsum_kernel");                                             \
+    const int rc2 = launch_status("importance_colsum_kernel");                                    \
+    if (rc2) return rc2;                                                                          \
+    hipLaunchKernelGGL(importance_reduce_kernel, grid3, dim3(256), 0, s, p);                      \
+    return launch_status("importance_reduce_kernel");                                             \
   }
   ACACHE_CASE(ACACHE_BF16, 128)
   ACACHE_CASE(ACACHE_BF16, 64)

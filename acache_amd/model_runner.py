@@ -437,8 +437,11 @@ class ModelRunner:
                 probe_shifts = self._to_device(shifts, torch.int32)
                 probe_sin, probe_cos = blocks[0].rotary_emb.get_rotary_embedding(
                     max(self._affix_relocation_max_position, max(shifts) + 1), self.device)
-            probe_scratch = torch.empty(max(16, 8 * int(probe_rows.numel()) * blocks[0].attn.num_heads),
-                                        dtype=torch.uint8, device=self.device)
+            probe_scratch = torch.empty(
+                max(16, ops.affix_importance_workspace_bytes(
+                    int(probe_rows.numel()), len(active_seqs), blocks[0].attn.num_heads, blocks[0].attn.num_kv_heads,
+                    blocks[0].attn.head_dim, affix_len, probe_shifts is not None)),
+                dtype=torch.uint8, device=self.device)
 
             def make_probe(layer_idx, block):
                 def probe(attention, q):

@@ -304,7 +304,7 @@ def affix_importance(
     shifts = _i32(affix_shifts, "affix_shifts") if relocate else None
     scale = softmax_scale if softmax_scale is not None else D ** -0.5
     lib = _lib.load()
-    need = lib.acache_affix_importance_workspace_bytes(total, H)
+    need = lib.acache_affix_importance_workspace_bytes(total, B, H, H_kv, D, affix_len, int(relocate))
     if workspace is None:
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     assert workspace.is_cuda and workspace.numel() * workspace.element_size() >= need
@@ -318,6 +318,14 @@ def affix_importance(
             _ptr(workspace), workspace.numel() * workspace.element_size(), _stream(q))
     _lib.check(rc, "affix_importance")
     return importance
+
+
+def affix_importance_workspace_bytes(total_mask_rows: int, batch: int, num_heads: int, num_kv_heads: int,
+                                     head_dim: int, affix_len: int, relocated: bool) -> int:
+    """Bytes of scratch ``affix_importance`` needs: row statistics, per-head partial sums and, when
+    ``affix_shifts`` are given, one re-rotated copy of the affix keys per request."""
+    return int(_lib.load().acache_affix_importance_workspace_bytes(
+        total_mask_rows, batch, num_heads, num_kv_heads, head_dim, affix_len, int(relocated)))
 
 
 def kv_scatter_layers(

@@ -267,10 +267,10 @@ def kernel_sweep(torch, device, ops, steps):
     cu_p = torch.arange(0, (B + 1) * M, M, dtype=torch.int32, device=device)
     sh_p = torch.randint(1, 256, (B,), generator=gen, device=device).to(torch.int32)
     imp = torch.zeros(B, A, dtype=torch.float32, device=device)
-    ws = torch.empty(8 * B * M * H, dtype=torch.uint8, device=device)
+    ws = torch.empty(ops.affix_importance_workspace_bytes(B * M, B, H, H, D, A, True), dtype=torch.uint8, device=device)
     us = timed(lambda: ops.affix_importance(imp, qp, kp, rows_p, cu_p, A, M, None, sh_p, cos, sin, 0, ws))
     flops = 2 * 2 * B * M * A * H * D   # the scores are computed twice (row statistics, then column sums)
-    out.append({"kernel": "importance_stats_kernel + importance_colsum_kernel", "us": round(us, 1),
+    out.append({"kernel": "importance kernels (rotate, stats, colsum, reduce)", "us": round(us, 1),
                 "TFLOPs": round(flops / us / 1e6, 1), "flops": flops,
                 "workload": "one layer: 16 requests x 256 mask queries x 1 000 affix keys, 32 heads x 128, bf16, key-side re-rotation"})
     logits = torch.randn(512, 126464, generator=gen, device=device).to(torch.bfloat16)

@@ -179,11 +179,13 @@ int acache_rope_qk_scatter(
  * dtype; here they are fp32.  Deterministic: no atomics, fixed summation order.
  *
  * mask_rows are row indices into q ([Tq, H, D] with the given strides).  workspace:
- * device scratch of at least acache_affix_importance_workspace_bytes(total_mask_rows, H)
- * bytes (row statistics between the two launches), 16-byte aligned, owned by the
- * caller.  max_mask_rows: an upper bound on the mask rows of one request.
+ * device scratch of at least acache_affix_importance_workspace_bytes(total_mask_rows, B, H,
+ * H_kv, D, affix_len, relocated = affix_shifts != NULL) bytes (row statistics, per-head
+ * partial sums and, with relocation, one re-rotated copy of the affix keys per request,
+ * passed between the launches), 16-byte aligned, owned by the caller.  max_mask_rows: an upper bound on the mask rows of one request.
  */
-int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_rows, int32_t H);
+int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_rows, int32_t B, int32_t H, int32_t H_kv,
+                                                int32_t D, int32_t affix_len, int32_t relocated);
 int acache_affix_importance(
     float *importance, const void *q, const void *k_cache,
     const int32_t *mask_rows, const int32_t *cu_mask, const int32_t *affix_shifts,
