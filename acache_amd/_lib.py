@@ -44,6 +44,9 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p]),
     "acache_block_table_slots": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int64, c_void_p]),
+    "acache_build_slot_layout": (c_int32, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        c_int32, c_int32, c_int32, c_int32, c_int64, c_void_p]),
     "acache_varlen_attn": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         c_float,

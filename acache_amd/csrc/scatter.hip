@@ -70,6 +70,63 @@ __global__ __launch_bounds__(256) void block_table_slots_kernel(
   }
 }
 
+// Slot layout of a batch of requests with a reused affix, one thread per token: where attention reads each
+// position from, and the (position, slot) list of the tokens that are recomputed (anchors + everything outside
+// the affix), in position order.  A request's private slots are enumerated block by block from its block table:
+// the first K go to its anchors in ascending position order, the rest to the non-affix positions in order.
+struct SlotLayoutParams {
+  int32_t *read_slots;
+  int32_t *recompute_pos;
+  int32_t *recompute_slots;
+  const int32_t *cu_len;
+  const int32_t *cu_rec;
+  const int32_t *affix_start;
+  const int32_t *affix_end;
+  const int32_t *cu_anchor;
+  const int32_t *anchors;
+  const int32_t *tables;
+  int32_t max_blocks;
+  int32_t block_size;
+  int32_t shared_slot_offset;
+};
+
+__global__ __launch_bounds__(256) void slot_layout_kernel(SlotLayoutParams p) {
+  const int b = blockIdx.y;
+  const int t0 = p.cu_len[b];
+  const int len = p.cu_len[b + 1] - t0;
+  const int a_lo = p.affix_start[b], a_hi = p.affix_end[b];
+  const int k0 = p.cu_anchor[b];
+  const int K = p.cu_anchor[b + 1] - k0;
+  const int r0 = p.cu_rec[b];
+  const int32_t *anc = p.anchors + k0;
+  for (int pos = blockIdx.x * 256 + threadIdx.x; pos < len; pos += gridDim.x * 256) {
+    int priv = -1, rank = -1;
+    if (pos >= a_lo && pos < a_hi) {
+      int lo = 0, hi = K;  // first anchor >= pos
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (anc[mid] < pos) lo = mid + 1; else hi = mid;
+      }
+      if (lo < K && anc[lo] == pos) { priv = lo; rank = a_lo + lo; }
+    } else if (pos < a_lo) {
+      priv = K + pos; rank = pos;
+    } else {
+      priv = K + pos - (a_hi - a_lo); rank = a_lo + K + (pos - a_hi);
+    }
+    int slot;
+    if (priv < 0) {
+      slot = p.shared_slot_offset + (pos - a_lo);  // frozen affix token: the shared copy
+    } else {
+      const int blk = priv / p.block_size;
+      const int id = blk < p.max_blocks ? p.tables[(int64_t)b * p.max_blocks + blk] : -1;
+      slot = id < 0 ? -1 : id * p.block_size + (priv - blk * p.block_size);
+      p.recompute_pos[r0 + rank] = pos;
+      p.recompute_slots[r0 + rank] = slot;
+    }
+    p.read_slots[t0 + pos] = slot;
+  }
+}
+
 }  // namespace acache
 
 using namespace acache;
@@ -124,4 +181,27 @@ extern "C" int acache_block_table_slots(
   hipLaunchKernelGGL(block_table_slots_kernel, dim3((unsigned)gx, (unsigned)B), dim3(256), 0,
                      (hipStream_t)stream, out_slots, block_tables, cu_k, B, max_blocks, block_size);
   return launch_status("block_table_slots_kernel");
+}
+
+extern "C" int acache_build_slot_layout(
+    int32_t *read_slots, int32_t *recompute_pos, int32_t *recompute_slots, const int32_t *cu_len,
+    const int32_t *cu_rec, const int32_t *affix_start, const int32_t *affix_end, const int32_t *cu_anchor,
+    const int32_t *anchors, const int32_t *block_tables, int32_t B, int32_t max_blocks, int32_t block_size,
+    int32_t shared_slot_offset, int64_t total_tokens, void *stream) {
+  if (B < 0 || max_blocks < 0 || block_size <= 0 || total_tokens < 0 || shared_slot_offset < 0)
+    return fail(ACACHE_E_SHAPE, "build_slot_layout: bad size");
+  if (B == 0 || total_tokens == 0) return 0;
+  if (!read_slots || !recompute_pos || !recompute_slots || !cu_len || !cu_rec || !affix_start || !affix_end ||
+      !cu_anchor || !block_tables)
+    return fail(ACACHE_E_NULL, "build_slot_layout: NULL pointer");
+  if (B > 65535) return fail(ACACHE_E_SHAPE, "build_slot_layout: batch %d > 65535", B);
+  int64_t gx = (total_tokens / B + 255) / 256 + 1;
+  if (gx > 1024) gx = 1024;
+  SlotLayoutParams p;
+  p.read_slots = read_slots; p.recompute_pos = recompute_pos; p.recompute_slots = recompute_slots;
+  p.cu_len = cu_len; p.cu_rec = cu_rec; p.affix_start = affix_start; p.affix_end = affix_end;
+  p.cu_anchor = cu_anchor; p.anchors = anchors; p.tables = block_tables;
+  p.max_blocks = max_blocks; p.block_size = block_size; p.shared_slot_offset = shared_slot_offset;
+  hipLaunchKernelGGL(slot_layout_kernel, dim3((unsigned)gx, (unsigned)B), dim3(256), 0, (hipStream_t)stream, p);
+  return launch_status("slot_layout_kernel");
 }

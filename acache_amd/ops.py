@@ -18,6 +18,7 @@ Additions with no single reference callable (documented at each function):
 from __future__ import annotations
 
 import math
+from itertools import accumulate as _accumulate
 
 import torch
 
@@ -326,6 +327,45 @@ def affix_importance_workspace_bytes(total_mask_rows: int, batch: int, num_heads
     ``affix_shifts`` are given, one re-rotated copy of the affix keys per request."""
     return int(_lib.load().acache_affix_importance_workspace_bytes(
         total_mask_rows, batch, num_heads, num_kv_heads, head_dim, affix_len, int(relocated)))
+
+
+def build_slot_layout(lengths, affix_spans, anchors, block_tables: torch.Tensor, block_size: int,
+                      shared_slot_offset: int = 0):
+    """Read slot maps and recompute lists of a batch in one launch (``Sequence.finalize_slot_mapping``,
+    nano-vdllm/sequence.py:169-202, for every request at once).
+
+    ``lengths``: tokens per request; ``affix_spans``: ``(start, end)`` per request; ``anchors``: ascending anchor
+    positions per request; ``block_tables``: int32 ``[B, max_blocks]`` on the device (-1 padded).
+    Returns ``(read_slots, recompute_pos, recompute_slots, cu_len, cu_rec)``, the first three int32 device tensors.
+    """
+    device = block_tables.device
+    B = len(lengths)
+    assert block_tables.is_cuda and block_tables.dtype == torch.int32 and block_tables.is_contiguous()
+    assert block_tables.shape[0] == B == len(affix_spans) == len(anchors)
+    rec = [len(a) + n - (e - s) for n, (s, e), a in zip(lengths, affix_spans, anchors)]
+    cu_len = [0] + list(_accumulate(lengths))
+    cu_rec = [0] + list(_accumulate(rec))
+    cu_anc = [0] + list(_accumulate(len(a) for a in anchors))
+    flat_anchors = [p for a in anchors for p in a]
+    meta = torch.tensor(cu_len + cu_rec + cu_anc + [s for s, _ in affix_spans] + [e for _, e in affix_spans]
+                        + (flat_anchors or [0]), dtype=torch.int32).to(device, non_blocking=True)
+    o = 0
+    parts = []
+    for n in (B + 1, B + 1, B + 1, B, B, max(len(flat_anchors), 1)):
+        parts.append(meta[o:o + n])
+        o += n
+    d_len, d_rec, d_anc, d_start, d_end, d_anchors = parts
+    read = torch.empty(cu_len[-1], dtype=torch.int32, device=device)
+    rpos = torch.empty(cu_rec[-1], dtype=torch.int32, device=device)
+    rslot = torch.empty(cu_rec[-1], dtype=torch.int32, device=device)
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        rc = lib.acache_build_slot_layout(
+            _ptr(read), _ptr(rpos) or read.data_ptr(), _ptr(rslot) or read.data_ptr(), _ptr(d_len), _ptr(d_rec),
+            _ptr(d_start), _ptr(d_end), _ptr(d_anc), _ptr(d_anchors), _ptr(block_tables), B, block_tables.shape[1],
+            block_size, shared_slot_offset, cu_len[-1], _stream(block_tables))
+    _lib.check(rc, "build_slot_layout")
+    return read, rpos, rslot, cu_len, cu_rec
 
 
 def kv_scatter_layers(

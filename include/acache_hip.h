@@ -255,6 +255,30 @@ int acache_block_table_slots(
     void *stream);
 
 /*
+ * Slot layout of a batch of requests that reuse a shared affix (device-side form of
+ * Sequence.finalize_slot_mapping, nano-vdllm/sequence.py:169-202, which the reference
+ * evaluates per request in Python before prepare_caching_acache,
+ * nano-vdllm/model_runner.py:1295-1471).
+ *
+ *   request b: tokens [0, len_b), affix [affix_start[b], affix_end[b]), anchors
+ *   anchors[cu_anchor[b] .. cu_anchor[b+1]) (ascending positions inside the affix),
+ *   private slot i = block_tables[b, i / block_size] * block_size + i % block_size.
+ *   The first K_b private slots belong to the anchors in position order, the rest to
+ *   the positions outside the affix in order.
+ *     read_slots[cu_len[b] + pos] = private slot of pos            (anchor or non-affix)
+ *                                 = shared_slot_offset + pos - affix_start[b]   (frozen affix)
+ *     recompute_pos / recompute_slots[cu_rec[b] + j]: the recomputed positions of b in
+ *     ascending order with their slots (K_b + len_b - affix_len_b entries).
+ */
+int acache_build_slot_layout(
+    int32_t *read_slots, int32_t *recompute_pos, int32_t *recompute_slots,
+    const int32_t *cu_len, const int32_t *cu_rec,
+    const int32_t *affix_start, const int32_t *affix_end,
+    const int32_t *cu_anchor, const int32_t *anchors,
+    const int32_t *block_tables, int32_t B, int32_t max_blocks, int32_t block_size,
+    int32_t shared_slot_offset, int64_t total_tokens, void *stream);
+
+/*
  * Bidirectional variable-length attention reading K/V through a slot map.
  *
  *   per request b, head h (kv head = h / (H / H_kv)):
