@@ -684,6 +684,7 @@ class ModelRunner:
         assert step > 0, "recompute_batch_size must be larger than 0"
         max_num_seqs = cfg.max_num_seqs if cfg.max_num_seqs > 0 else len(prompts)
         use_acache = prefix is not None
+        dream = str(getattr(cfg, "model_type", "")).lower() == "dream"
         if timing is None:
             timing = self._new_timing(mode, len(prompts))
         self.last_timing = timing or {}
@@ -733,6 +734,15 @@ class ModelRunner:
                 else:
                     input_ids, positions, gen_starts, current = self.prepare_caching(batch, part)
                     keep = gen_starts.unsqueeze(1) + block_length * current.unsqueeze(1) + offsets
+                if dream:
+                    # Dream reads token i from the hidden state of the row in front of it (the first row of a
+                    # request keeps its own): model_runner.py:63-66
+                    group = self._select(batch, part)
+                    if use_acache:
+                        first = block_starts - self._to_device([s.block_query_start() for s in group], torch.int32)
+                    else:
+                        first = gen_starts - self._to_device([s.generation_start for s in group], torch.int32)
+                    keep = torch.maximum(keep, first.unsqueeze(1) + 1) - 1
                 self._finish_timing(timing, "cache_prepare", start)
                 start = self._start_timing()
                 logits = model(input_ids, position_ids=positions, logits_keep_indices=keep.flatten().long()).logits
@@ -741,11 +751,15 @@ class ModelRunner:
                 self._add_timing_count(timing, "cache_forward_nfe", len(part))
                 start = self._start_timing()
                 logits = logits.view(len(part), block_length, -1)
-                current_blocks = working[part]
-                x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
-                                                       current_blocks, threshold)
-                r, c = torch.where(transfer)
-                working[part[r], c] = x0[transfer]
+                if dream:
+                    # a refresh commits only the first token of the block (model_runner.py:68-78, 1548-1552)
+                    working[part, 0] = self._sample_dream_seed_tokens(logits[:, 0])
+                else:
+                    current_blocks = working[part]
+                    x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
+                                                           current_blocks, threshold)
+                    r, c = torch.where(transfer)
+                    working[part[r], c] = x0[transfer]
                 self._finish_timing(timing, "cache_update", start)
             total_nfe += len(rows)
 
@@ -816,6 +830,8 @@ class ModelRunner:
                     graph.replay()
                 else:
                     logits = model(working[active], position_ids=decoding_positions).logits
+                if dream:  # block-local shift: position i is predicted by the row in front of it (56-61)
+                    logits = torch.cat([logits[:, :1], logits[:, :-1]], dim=1)
                 self._finish_timing(timing, "decode_forward", start)
                 self._add_timing_count(timing, "decode_forward_calls", 1)
                 self._add_timing_count(timing, "decode_forward_nfe", len(active))
@@ -855,6 +871,13 @@ class ModelRunner:
         with torch.cuda.graph(graph):
             logits = self.model(static_tokens, position_ids=positions).logits
         return graph, static_tokens, logits
+
+    def _sample_dream_seed_tokens(self, logits):
+        """First token of a freshly refreshed block: arg-max, or a categorical draw at temperature > 0."""
+        temperature = float(self.config.temperature)
+        if temperature > 0:
+            return torch.distributions.Categorical(probs=torch.softmax(logits.float() / temperature, dim=-1)).sample()
+        return logits.argmax(dim=-1)
 
     # ------------------------------------------------------------------ token transfer (2279-2314)
     def get_transfer_index(self, logits, temperature, remasking, mask_index, x, threshold=0.9):

@@ -113,3 +113,41 @@ def test_dream_hf_layout_affix_cache(device):
     with pytest.raises(ValueError, match="does not match"):
         GD.generate_with_anchor_attention(model, torch.tensor([prompt], device=device), precomputed_affix_cache=cache,
                                           **{**args, "affix_end": 31})
+
+
+def test_batched_engine_applies_the_dream_rule(device):
+    """ModelRunner with model_type='dream' (model_runner.py:56-78, 1525-1552, 1703): shifted keep indices at a
+    refresh, first-token seeding, block-shifted refinement logits.  For a single request it must commit the tokens
+    of the HF-signature Dream entry point, with and without affix reuse."""
+    from acache_amd.config import Config
+    from acache_amd.model_runner import ModelRunner
+    from acache_amd.sequence import Sequence
+    cfg, model = _model(device, seed=9)
+    affix = list(range(10, 26))
+    prompt = [3, 4] + affix + [5, 6, 7]
+    want, _ = GD.generate_with_anchor_attention(
+        model, torch.tensor([prompt], device=device), steps=8, gen_length=8, block_length=4, mask_id=MASK,
+        threshold=0.9, anchor_ratio=0.25, affix_start=2, affix_end=18)
+    serve = Config(hf_config=cfg, mask_id=MASK, recompute_batch_size=1, max_num_seqs=1, gen_length=8, block_length=4,
+                   threshold=0.9, cache_block_size=256, num_kvcache_blocks=8, temperature=0.0, enable_acache=True,
+                   anchor_ratio=0.25, model_type="dream")
+    runner = ModelRunner(model, serve)
+    seq = Sequence(list(prompt), gen_length=8, block_length=4, cache_block_size=256, mask_id=MASK,
+                   prompt_affix_start=2, prompt_affix_end=18)
+    out, nfe = runner.generate_with_acache([seq])
+    assert out[0] == want[0, -8:].tolist()
+    # full recompute on the same weights: every position is predicted from its left neighbour too
+    base = ModelRunner(model, Config(hf_config=cfg, mask_id=MASK, recompute_batch_size=1, max_num_seqs=1, gen_length=8,
+                                     block_length=4, threshold=0.9, cache_block_size=256, num_kvcache_blocks=8,
+                                     temperature=0.0, enable_acache=False, model_type="dream"))
+    seq_b = Sequence(list(prompt), gen_length=8, block_length=4, cache_block_size=256, mask_id=MASK)
+    out_b, _ = base.generate_with_dual_cache([seq_b])
+    assert len(out_b[0]) == 8 and MASK not in out_b[0]
+    # anchor_ratio 1.0 recomputes the whole affix: ACache must then agree with full recompute (bf16 noise aside)
+    full = ModelRunner(model, Config(hf_config=cfg, mask_id=MASK, recompute_batch_size=1, max_num_seqs=1, gen_length=8,
+                                     block_length=4, threshold=0.9, cache_block_size=256, num_kvcache_blocks=8,
+                                     temperature=0.0, enable_acache=True, anchor_ratio=1.0, model_type="dream"))
+    seq_f = Sequence(list(prompt), gen_length=8, block_length=4, cache_block_size=256, mask_id=MASK,
+                     prompt_affix_start=2, prompt_affix_end=18)
+    out_f, _ = full.generate_with_acache([seq_f])
+    assert sum(a == b for a, b in zip(out_f[0], out_b[0])) >= 6
