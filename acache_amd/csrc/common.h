@@ -67,6 +67,14 @@ __device__ __forceinline__ void store16_stream(void *p, const vec16 &v) {
   u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
   __builtin_nontemporal_store(t, reinterpret_cast<u4 *>(p));
 }
+// Write-through streaming store (nt sc0 sc1): the line goes to memory without being kept in L2 or the
+// Infinity Cache.  For the relocation output, 9 GB written once per launch, this measured 2 % faster than
+// the plain non-temporal store.
+__device__ __forceinline__ void store16_writethrough(void *p, const vec16 &v) {
+  typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+  const u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
+  asm volatile("global_store_dwordx4 %0, %1, off nt sc0 sc1" ::"v"(p), "v"(t) : "memory");
+}
 
 // ------------------------------------------------------- element <-> fp32 ----
 // bf16 is handled as raw bits so rounding is exactly round-to-nearest-even with

@@ -129,10 +129,10 @@ __global__ __launch_bounds__(256) void relocate_kernel(RelocateParams p) {
       }
       char *kd = p.out_k + (int64_t)(l0 + i) * p.out_layer_bytes + dst_off;
       char *vd = p.out_v + (int64_t)(l0 + i) * p.out_layer_bytes + dst_off;
-      store16_stream(kd, k_lo[i]);
-      store16_stream(kd + HALF_BYTES, k_hi[i]);
-      store16_stream(vd, v_lo[i]);
-      store16_stream(vd + HALF_BYTES, v_hi[i]);
+      store16_writethrough(kd, k_lo[i]);
+      store16_writethrough(kd + HALF_BYTES, k_hi[i]);
+      store16_writethrough(vd, v_lo[i]);
+      store16_writethrough(vd + HALF_BYTES, v_hi[i]);
     }
   }
 }
