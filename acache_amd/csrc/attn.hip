@@ -6,19 +6,24 @@
 //   keys in tiles of BN = 64, staged through LDS and shared by the 4 waves.
 //
 // MFMA formulation (v_mfma_f32_16x16x32, 64-wide wavefronts)
-//   S^T = K Q^T   : A = K tile rows (LDS, row-major, padded pitch), B = Q (registers)
-//   O^T = V^T P^T : A = V^T (LDS, transposed + XOR-swizzled on the way in),
-//                   B = P^T, which is exactly the accumulator layout of S^T after
-//                   a bf16 pack — probabilities never leave registers.
-//   In both products a lane owns ONE query column, so the running max, the
-//   rescale factor and the running sum are per-lane scalars; the only cross-lane
-//   traffic of the softmax is two xor-shuffles per tile for the row maximum.
+//   S^T = K Q^T   : A = K tile rows from LDS, B = Q (registers)
+//   O^T = V^T P^T : A = V^T from LDS, B = P^T, which is exactly the accumulator
+//                   layout of S^T after a bf16 pack — probabilities never leave
+//                   registers.
+//   In both products a lane owns ONE query column, so the running maximum and the
+//   rescale factor are per-lane scalars; the softmax denominator is one more
+//   MFMA row block (V^T rows of ones).
 //
-// K/V rows are fetched through the slot map (16 lanes x 16 B per 256-byte row),
-// optionally re-rotated on the key side, and prefetched into registers one tile
-// ahead of the MFMA work.  HBM traffic per call: K and V rows once per
-// (request, kv head) when query tiles of one head share an L2 (the block index
-// is remapped so that they land on the same XCD), Q once, O once.
+// Two kernels:
+//   varlen_attn_dma_kernel (plain and query-side relocation): K/V rows are copied
+//     global -> LDS directly through the slot map into a two-deep ring, swizzled by
+//     permuting the global side of the copy; V stays row-major and is read with
+//     the LDS transpose read.
+//   varlen_attn_kernel (key-side relocation): rows are staged through registers,
+//     re-rotated there, and V is transposed on the way into LDS.
+// Both share the softmax steps below, so they round identically.  HBM traffic per
+// call: K and V rows once per (request, kv head) when query tiles of one head share
+// an L2 (block indices are mapped so that they land on the same XCD), Q once, O once.
 #include "common.h"
 #include "mma.h"
 
@@ -91,8 +96,6 @@ __device__ __forceinline__ bool locate_query_tile(const int32_t *cu_q, int B, in
   return false;
 }
 
-// Key range of tile t: the shared range [0, shared_len) comes first in tiles of BN
-// (query-side mode only, otherwise shared_len = 0), then [shared_len, kv_len).
 // Same lookup, but over the requests sorted by descending key count (ties: lower index first), for
 // batches of up to 64 requests.  A block's run time is proportional to its request's key count
 // and the hardware hands out blocks in index order, so this is longest-processing-time-first
@@ -121,6 +124,8 @@ __device__ __forceinline__ bool locate_query_tile_lpt(const int32_t *cu_q, const
   return true;
 }
 
+// Key range of tile t: the shared range [0, shared_len) comes first in tiles of BN
+// (query-side mode only, otherwise shared_len = 0), then [shared_len, kv_len).
 struct TileRange {
   int n0, n_end;
 };

@@ -400,7 +400,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; --gpus N with N > 1 is not supported "
-              "(the path shards by request or KV head without communication, see DESIGN.md)", file=sys.stderr)
+              "(the path shards by request or by KV head without communication between GPUs)", file=sys.stderr)
         sys.exit(2)
 
     import torch
