@@ -28,7 +28,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 # HBM bytes per launch of the default workloads, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # script (raw counters scaled by what they read for the 1 GiB copy of --copy-calibration: x2.000 and x1.000);
 # the summaries with the commands are profiles/relocate_kernel_*.md and profiles/varlen_attn_dma_kernel_*.md.
-MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 17.991e9, "attention": 284.2e6}
+MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 18.029e9, "attention": 284.5e6}
 
 
 def _event_times_ms(fn, steps, torch):

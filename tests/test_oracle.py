@@ -394,3 +394,61 @@ def test_affix_importance_closed_forms_and_brute_force():
     same[:] = kc[0]
     u = O.affix_importance(q, same, mask_rows, cu, A)
     assert torch.allclose(u[0], torch.full((A,), 3.0 * H / A), atol=1e-5)
+
+
+# ------------------------------------------------------------------ fused rotary + scatter (modeling_llada.py:412-453, attention.py:22-41)
+def test_rope_qk_scatter_is_rotation_at_positions_then_scatter():
+    g = torch.Generator().manual_seed(5)
+    N, H, Hkv, D = 7, 4, 2, 64
+    cos, sin = O.rope_table(32, D, 1e4)
+    q = torch.randn(N, H, D, generator=g, dtype=torch.float64)
+    k = torch.randn(N, Hkv, D, generator=g, dtype=torch.float64)
+    v = torch.randn(N, Hkv, D, generator=g, dtype=torch.float64)
+    pos = torch.tensor([0, 3, 3, 31, 7, 1, 20])
+    slots = torch.tensor([5, -1, 0, 9, 2, -1, 7], dtype=torch.int32)
+    kc = torch.full((12, Hkv, D), 7.0, dtype=torch.float64)
+    vc = torch.full((12, Hkv, D), 7.0, dtype=torch.float64)
+    q_rot, k_rot = O.rope_qk_scatter(q, k, v, pos, cos.double(), sin.double(), kc, vc, slots)
+    # explicit 2x2 rotation of every (d, d + D/2) pair by pos * theta^(-2d/D), in float64
+    inv = 1e4 ** (-torch.arange(0, D, 2, dtype=torch.float64) / D)
+    ang = pos.double()[:, None] * inv[None, :]
+    for x, y in ((q, q_rot), (k, k_rot)):
+        lo, hi = x[..., :D // 2], x[..., D // 2:]
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        want = torch.cat((lo * c - hi * s, hi * c + lo * s), dim=-1)
+        assert torch.allclose(y, want, atol=1e-6)          # the tables are fp32
+    assert torch.equal(q_rot[0], q[0]) and torch.equal(k_rot[0], k[0])   # position 0: identity
+    # the cache holds the rotated k and the plain v at the mapped slots, nothing else moved
+    for i, s in enumerate(slots.tolist()):
+        if s >= 0:
+            assert torch.equal(kc[s], k_rot[i]) and torch.equal(vc[s], v[i])
+    untouched = [s for s in range(12) if s not in slots.tolist()]
+    assert (kc[untouched] == 7.0).all() and (vc[untouched] == 7.0).all()
+    # without a slot map nothing is written
+    kc2 = kc.clone()
+    O.rope_qk_scatter(q, k, v, pos, cos.double(), sin.double(), kc2, vc, None)
+    assert torch.equal(kc2, kc)
+
+
+# ------------------------------------------------------------------ token and confidence (model_runner.py:2279-2296)
+def test_argmax_confidence_against_float64_softmax_and_edge_rows():
+    g = torch.Generator().manual_seed(6)
+    logits = (torch.randn(5, 3, 97, generator=g) * 4).to(torch.bfloat16)
+    tok, conf = O.argmax_confidence(logits)
+    p = torch.softmax(logits.double(), dim=-1)
+    assert tok.shape == conf.shape == (5, 3)
+    assert torch.equal(tok, p.argmax(-1))
+    assert torch.allclose(conf.double(), p.max(-1).values, rtol=1e-5)
+    # given picks: their probability, the picks handed back
+    picks = torch.randint(0, 97, (5, 3), generator=g)
+    tok2, conf2 = O.argmax_confidence(logits, picks)
+    assert torch.equal(tok2, picks)
+    assert torch.allclose(conf2.double(), p.gather(-1, picks[..., None]).squeeze(-1), rtol=1e-5)
+    # ties go to the first maximum; a one-hot row has confidence 1; a uniform row 1/V
+    rows = torch.zeros(3, 8)
+    rows[0, 2] = rows[0, 5] = 3.0
+    rows[1, 6] = 200.0
+    tok3, conf3 = O.argmax_confidence(rows)
+    assert tok3.tolist() == [2, 6, 0]
+    assert abs(float(conf3[1]) - 1.0) < 1e-6 and abs(float(conf3[2]) - 1 / 8) < 1e-7
+    assert abs(float(conf3[0]) - math.exp(3) / (2 * math.exp(3) + 6)) < 1e-6
