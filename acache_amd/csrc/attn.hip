@@ -55,6 +55,7 @@ struct AttnParams {
   int32_t H;
   int32_t H_kv;
   int32_t num_tiles;  // upper bound on the number of BM-row query tiles
+  int32_t head_dim;   // real head_dim (read by the padded any-head_dim variant only)
   int64_t num_slots;
   int64_t q_token_bytes, q_head_bytes;
   int64_t o_token_bytes, o_head_bytes;
@@ -222,8 +223,13 @@ __device__ __forceinline__ void softmax_probs_slab(const f32x4 (&s_acc)[NQ16][NT
   }
 }
 
-template <int DTYPE, int D, int NQ16, int MODE>
-__global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
+//
+// RAGGED = true is the any-head_dim variant: D is then the padded width (a multiple of 32) and the real
+// head_dim (a multiple of 16, at most D) comes in p.head_dim.  Rows are laid out in LDS at their real
+// width, the padding columns are zeroed once and never written again, and every loop over k-slabs and
+// d tiles skips the ones past the real width with a wave-uniform test.  Same arithmetic per element.
+template <int DTYPE, int D, int NQ16, int MODE, bool RAGGED = false>
+__global__ __launch_bounds__(256, RAGGED ? 1 : 2) void varlen_attn_kernel(AttnParams p) {
   constexpr int BN = 64;
   constexpr int WQ = 16 * NQ16;
   constexpr int BM = 4 * WQ;
@@ -234,15 +240,23 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
   constexpr int ROW_BYTES = D * 2;
   constexpr int CH = ROW_BYTES / 16;    // 16-byte chunks per row
   constexpr int PP = CH / 2;            // chunk pairs per row (K loader)
-  constexpr int K_ROWS_PER_PASS = 256 / PP;
-  constexpr int K_PASSES = BN / K_ROWS_PER_PASS;
-  constexpr int KPITCH = ROW_BYTES + 16;
-  constexpr int V_THREADS = CH * (BN / 4);  // one thread per (chunk, 4-row group)
+  constexpr int K_PAIRS = BN * PP;      // one thread per (row, chunk pair) and pass
+  constexpr int K_PASSES = (K_PAIRS + 255) / 256;
+  // the padded variant swizzles the chunks of a K row instead of padding the pitch (64 KiB of LDS at D = 256)
+  constexpr int KPITCH = RAGGED ? ROW_BYTES : ROW_BYTES + 16;
+  constexpr int V_ITEMS = CH * (BN / 4);  // one thread per (chunk, 4-row group) and pass
+  constexpr int V_PASSES = (V_ITEMS + 255) / 256;
   constexpr int VPITCH = BN * 2;            // bytes per V^T row (swizzled, unpadded)
   using M = Mma<DTYPE>;
 
   __shared__ __attribute__((aligned(16))) char lds_k[BN * KPITCH];
   __shared__ __attribute__((aligned(16))) char lds_v[D * VPITCH];
+
+  const int d_real = RAGGED ? p.head_dim : D;
+  const int ch_real = d_real / 8;       // 16-byte chunks of a real row
+  const int pp_real = ch_real / 2;      // the rotate-half partner of chunk c is chunk c + pp_real
+  // position of chunk c of K row r inside its LDS row
+  auto kpos = [](int r, int c) __attribute__((always_inline)) { return RAGGED ? (c ^ (r & 15)) : c; };
 
   // ---- which (request, query tile, head) is this workgroup? -----------------
   const int per_xcd = gridDim.x >> 3;
@@ -275,7 +289,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
   if (kv_len <= 0) {  // no keys: defined output (zeros)
     for (int r = tid / CH; r < BM; r += 256 / CH) {
       const int qr = q_tile0 + r;
-      if (qr < q_len) store16(out_base + (int64_t)qr * p.o_token_bytes + (tid % CH) * 16, vec16{{0, 0, 0, 0}});
+      if (qr < q_len && tid % CH < ch_real)
+        store16(out_base + (int64_t)qr * p.o_token_bytes + (tid % CH) * 16, vec16{{0, 0, 0, 0}});
     }
     return;
   }
@@ -298,10 +313,11 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
     const bool live = qr < q_len;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      qf[qt][ks] = live ? load16(q_base + (int64_t)qr * p.q_token_bytes + (32 * ks + 8 * lg) * 2)
-                        : vec16{{0, 0, 0, 0}};
+      qf[qt][ks] = live && 32 * ks + 8 * lg < d_real
+                       ? load16(q_base + (int64_t)qr * p.q_token_bytes + (32 * ks + 8 * lg) * 2)
+                       : vec16{{0, 0, 0, 0}};
     }
-    if (MODE == MODE_QUERY_SIDE) {
+    if (MODE == MODE_QUERY_SIDE && !RAGGED) {
       const float *cr = p.cos_tab + (int64_t)shift * D;
       const float *sr = p.sin_tab + (int64_t)shift * D;
 #pragma unroll
@@ -312,48 +328,85 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
         qs[qt][ks + KS / 2] = hi;
       }
     }
+    if (MODE == MODE_QUERY_SIDE && RAGGED) {
+      // the partner chunk (d +- head_dim/2) belongs to another lane here: fetch it, rotate the pair, keep our half
+      const float *cr = p.cos_tab + (int64_t)shift * d_real;
+      const float *sr = p.sin_tab + (int64_t)shift * d_real;
+      const int half = d_real / 2;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d0 = 32 * ks + 8 * lg;
+        qs[qt][ks] = qf[qt][ks];
+        if (live && d0 < d_real && shift != 0) {
+          const bool first = d0 < half;
+          const int dl = first ? d0 : d0 - half;
+          const vec16 other = load16(q_base + (int64_t)qr * p.q_token_bytes + (first ? d0 + half : dl) * 2);
+          vec16 lo = first ? qf[qt][ks] : other, hi = first ? other : qf[qt][ks];
+          rotate_pair_half<DTYPE>(lo, hi, cr, sr, dl, half, -1.0f);
+          qs[qt][ks] = first ? lo : hi;
+        }
+      }
+    }
   }
 
   // ---- loader state ------------------------------------------------------------
-  // K: thread -> (row kr + pass*K_ROWS_PER_PASS, chunk pair kc / kc + PP)
-  const int kr = tid / PP, kc = tid % PP;
-  // V: thread -> (chunk vc, rows 4*vrg .. 4*vrg+3); threads >= V_THREADS idle
-  const int vc = tid % CH, vrg = tid / CH;
-  const bool v_thread = tid < V_THREADS;
-  vec16 k_lo[K_PASSES], k_hi[K_PASSES], v_row[4];
+  // K: thread -> (row kr0 + pass * K_ROWS_PER_PASS, chunk pair kc / kc + pp_real)
+  // V: thread -> (chunk vc, rows 4*vrg .. 4*vrg+3 with vrg = vrg0 + pass * V_GROUPS_PER_PASS)
+  // row groups past the tile, and chunks past the real row width, stay idle
+  static_assert(256 % PP == 0 && K_PAIRS % 256 == 0 && 256 % CH == 0, "the loaders want a power-of-two row width");
+  constexpr int K_ROWS_PER_PASS = 256 / PP;
+  constexpr int V_GROUPS_PER_PASS = 256 / CH;
+  const int kr0 = tid / PP, kc = tid % PP;
+  const int vc = tid % CH, vrg0 = tid / CH;
+  const bool k_thread = !RAGGED || kc < pp_real;
+  vec16 k_lo[K_PASSES], k_hi[K_PASSES], v_row[V_PASSES][4];
   const char *kc_base = p.k_cache + (int64_t)kvh * p.kv_head_bytes;
   const char *vc_base = p.v_cache + (int64_t)kvh * p.kv_head_bytes;
+  auto v_live = [&](int vrg) __attribute__((always_inline)) {
+    return (V_ITEMS % 256 == 0 || vrg < BN / 4) && (!RAGGED || vc < ch_real);
+  };
+
+  if (RAGGED) {  // the padding columns of both tiles are zero for the whole kernel
+    for (int i = tid * 16; i < BN * KPITCH; i += 256 * 16) store16(lds_k + i, vec16{{0, 0, 0, 0}});
+    for (int i = tid * 16; i < D * VPITCH; i += 256 * 16) store16(lds_v + i, vec16{{0, 0, 0, 0}});
+    __syncthreads();
+  }
 
   auto fetch = [&](int n0, int n_end) __attribute__((always_inline)) {
 #pragma unroll
     for (int ps = 0; ps < K_PASSES; ++ps) {
-      const int n = n0 + kr + ps * K_ROWS_PER_PASS;
+      const int n = n0 + kr0 + ps * K_ROWS_PER_PASS;
       k_lo[ps] = vec16{{0, 0, 0, 0}};
       k_hi[ps] = k_lo[ps];
-      if (n < n_end) {
+      if (k_thread && n < n_end) {
         const int64_t slot = p.slot_map[kv_begin + n];
         if (slot >= 0 && slot < p.num_slots) {
           const char *src = kc_base + slot * p.kv_slot_bytes + kc * 16;
           k_lo[ps] = load16(src);
-          k_hi[ps] = load16(src + ROW_BYTES / 2);
+          k_hi[ps] = load16(src + pp_real * 16);
           if (MODE == MODE_KEY_SIDE && slot < p.shared_prefix_len) {
             const int delta = n - (int)slot;
             const int ad = delta < 0 ? -delta : delta;
             if (delta != 0 && ad < p.rope_rows)
-              rotate_pair<DTYPE, D>(k_lo[ps], k_hi[ps], p.cos_tab + (int64_t)ad * D,
-                                    p.sin_tab + (int64_t)ad * D, kc * 8, delta < 0 ? -1.0f : 1.0f);
+              rotate_pair_half<DTYPE>(k_lo[ps], k_hi[ps], p.cos_tab + (int64_t)ad * d_real,
+                                      p.sin_tab + (int64_t)ad * d_real, kc * 8, d_real / 2,
+                                      delta < 0 ? -1.0f : 1.0f);
           }
         }
       }
     }
-    if (v_thread) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = n0 + 4 * vrg + r;
-        v_row[r] = vec16{{0, 0, 0, 0}};
-        if (n < n_end) {
-          const int64_t slot = p.slot_map[kv_begin + n];
-          if (slot >= 0 && slot < p.num_slots) v_row[r] = load16(vc_base + slot * p.kv_slot_bytes + vc * 16);
+    for (int ps = 0; ps < V_PASSES; ++ps) {
+      const int vrg = vrg0 + ps * V_GROUPS_PER_PASS;
+      if (v_live(vrg)) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = n0 + 4 * vrg + r;
+          v_row[ps][r] = vec16{{0, 0, 0, 0}};
+          if (n < n_end) {
+            const int64_t slot = p.slot_map[kv_begin + n];
+            if (slot >= 0 && slot < p.num_slots) v_row[ps][r] = load16(vc_base + slot * p.kv_slot_bytes + vc * 16);
+          }
         }
       }
     }
@@ -362,32 +415,39 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
   auto stage = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int ps = 0; ps < K_PASSES; ++ps) {
-      char *dst = lds_k + (kr + ps * K_ROWS_PER_PASS) * KPITCH + kc * 16;
-      store16(dst, k_lo[ps]);
-      store16(dst + ROW_BYTES / 2, k_hi[ps]);
+      const int kr = kr0 + ps * K_ROWS_PER_PASS;
+      if (k_thread) {
+        char *dst = lds_k + kr * KPITCH;
+        store16(dst + kpos(kr, kc) * 16, k_lo[ps]);
+        store16(dst + kpos(kr, kc + pp_real) * 16, k_hi[ps]);
+      }
     }
-    if (v_thread) {
-      // 4 rows x 8 elements -> 8 columns x 4 keys; key n sits at position
-      // 32*(n/32) + 8*((n%16)/4) + 4*((n%32)/16) + n%4 inside its V^T row, the
-      // order in which the S^T accumulator hands probabilities to the PV product
-      const int n4 = 4 * vrg;
-      const int chunk = 4 * (n4 >> 5) + ((n4 & 15) >> 2);
-      const int half = (n4 & 31) >> 4;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int d = 8 * vc + j;
-        const uint32_t w0 = v_row[0].w[j >> 1], w1 = v_row[1].w[j >> 1];
-        const uint32_t w2 = v_row[2].w[j >> 1], w3 = v_row[3].w[j >> 1];
-        uint2 val;
-        if (j & 1) {
-          val.x = (w0 >> 16) | (w1 & 0xffff0000u);
-          val.y = (w2 >> 16) | (w3 & 0xffff0000u);
-        } else {
-          val.x = (w0 & 0xffffu) | (w1 << 16);
-          val.y = (w2 & 0xffffu) | (w3 << 16);
+    for (int ps = 0; ps < V_PASSES; ++ps) {
+      const int vrg = vrg0 + ps * V_GROUPS_PER_PASS;
+      if (v_live(vrg)) {
+        // 4 rows x 8 elements -> 8 columns x 4 keys; key n sits at position
+        // 32*(n/32) + 8*((n%16)/4) + 4*((n%32)/16) + n%4 inside its V^T row, the
+        // order in which the S^T accumulator hands probabilities to the PV product
+        const int n4 = 4 * vrg;
+        const int chunk = 4 * (n4 >> 5) + ((n4 & 15) >> 2);
+        const int half = (n4 & 31) >> 4;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int d = 8 * vc + j;
+          const uint32_t w0 = v_row[ps][0].w[j >> 1], w1 = v_row[ps][1].w[j >> 1];
+          const uint32_t w2 = v_row[ps][2].w[j >> 1], w3 = v_row[ps][3].w[j >> 1];
+          uint2 val;
+          if (j & 1) {
+            val.x = (w0 >> 16) | (w1 & 0xffff0000u);
+            val.y = (w2 >> 16) | (w3 & 0xffff0000u);
+          } else {
+            val.x = (w0 & 0xffffu) | (w1 << 16);
+            val.y = (w2 & 0xffffu) | (w3 << 16);
+          }
+          const int swz = ((d >> 1) & 7) ^ ((d >> 4) & 7);
+          *reinterpret_cast<uint2 *>(lds_v + d * VPITCH + ((chunk ^ swz) << 4) + (half << 3)) = val;
         }
-        const int swz = ((d >> 1) & 7) ^ ((d >> 4) & 7);
-        *reinterpret_cast<uint2 *>(lds_v + d * VPITCH + ((chunk ^ swz) << 4) + (half << 3)) = val;
       }
     }
   };
@@ -439,7 +499,8 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
       for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const vec16 kf = load16(lds_k + (16 * nt + li) * KPITCH + (4 * ks + lg) * 16);
+          if (RAGGED && 32 * ks >= d_real) continue;
+          const vec16 kf = load16(lds_k + (16 * nt + li) * KPITCH + kpos(li, 4 * ks + lg) * 16);
 #pragma unroll
           for (int qt = 0; qt < NQ16; ++qt)
             s_acc[qt][nt] = M::run(kf, qq[qt][ks], s_acc[qt][nt]);
@@ -459,6 +520,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
     // O^T += V^T P^T ; lane reads V^T[16*dt + li][keys of slab s, group lg]
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+      if (RAGGED && 16 * dt >= d_real) continue;
       const int d = 16 * dt + li;
       const int swz = ((d >> 1) & 7) ^ ((d >> 4) & 7);
 #pragma unroll
@@ -484,6 +546,7 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_kernel(AttnParams p) {
         char *dst = out_base + (int64_t)qr * p.o_token_bytes + 4 * lg * 2;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
+          if (RAGGED && 16 * dt >= d_real) continue;
           uint2 val;
           val.x = M::pack2(o_acc[qt][dt][0] * inv, o_acc[qt][dt][1] * inv);
           val.y = M::pack2(o_acc[qt][dt][2] * inv, o_acc[qt][dt][3] * inv);
@@ -935,6 +998,32 @@ static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStrea
   return launch_status("varlen_attn_kernel");
 }
 
+// Any other head_dim (a multiple of 16 up to 256): the register-staged kernel at a padded width of 256,
+// 16 query rows per wave, all three relocation modes.  A correctness path for model shapes outside the two
+// tuned widths, not a tuned one.
+template <int DTYPE>
+static int launch_attn_any_head_dim(const AttnParams &p0, int mode, int64_t total_q, hipStream_t stream) {
+  AttnParams p = p0;
+  constexpr int BM = 64, DPAD = 256;
+  p.num_tiles = (int32_t)((total_q + BM - 1) / BM) + p.B;
+  int64_t blocks = (int64_t)p.num_tiles * p.H;
+  blocks = (blocks + 7) / 8 * 8;
+  if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
+  dim3 grid((unsigned)blocks), block(256);
+  switch (mode) {
+    case MODE_PLAIN:
+      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, DPAD, 1, MODE_PLAIN, true>), grid, block, 0, stream, p);
+      break;
+    case MODE_KEY_SIDE:
+      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, DPAD, 1, MODE_KEY_SIDE, true>), grid, block, 0, stream, p);
+      break;
+    default:
+      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, DPAD, 1, MODE_QUERY_SIDE, true>), grid, block, 0, stream, p);
+      break;
+  }
+  return launch_status("varlen_attn_kernel (any head_dim)");
+}
+
 }  // namespace acache
 
 using namespace acache;
@@ -949,7 +1038,8 @@ extern "C" int acache_varlen_attn(
     int64_t kv_head_stride, void *stream) {
   if (dtype != ACACHE_BF16 && dtype != ACACHE_F16)
     return fail(ACACHE_E_DTYPE, "varlen_attn: dtype %d not supported (bf16 or f16)", dtype);
-  if (D != 128 && D != 64) return fail(ACACHE_E_SHAPE, "varlen_attn: head_dim %d not supported (64 or 128)", D);
+  if (D < 16 || D > 256 || D % 16 != 0)
+    return fail(ACACHE_E_SHAPE, "varlen_attn: head_dim %d not supported (a multiple of 16 up to 256)", D);
   if (B < 0 || total_q < 0 || total_k < 0 || H <= 0 || H_kv <= 0 || H % H_kv != 0 || num_slots < 0)
     return fail(ACACHE_E_SHAPE, "varlen_attn: bad sizes (H=%d, H_kv=%d)", H, H_kv);
   if (!(scale > 0.0f) || scale > 3.0e38f)
@@ -975,7 +1065,7 @@ extern "C" int acache_varlen_attn(
   p.cos_tab = rope_cos; p.sin_tab = rope_sin;
   p.scale_log2e = scale * 1.4426950408889634f;
   p.shared_prefix_len = relocate ? shared_prefix_len : 0;
-  p.rope_rows = rope_rows; p.B = B; p.H = H; p.H_kv = H_kv; p.num_tiles = 0;
+  p.rope_rows = rope_rows; p.B = B; p.H = H; p.H_kv = H_kv; p.num_tiles = 0; p.head_dim = D;
   p.num_slots = num_slots;
   p.q_token_bytes = q_token_stride * es; p.q_head_bytes = q_head_stride * es;
   p.o_token_bytes = out_token_stride * es; p.o_head_bytes = out_head_stride * es;
@@ -989,5 +1079,6 @@ extern "C" int acache_varlen_attn(
   ACACHE_ATTN(ACACHE_F16, 128)
   ACACHE_ATTN(ACACHE_F16, 64)
 #undef ACACHE_ATTN
-  return fail(ACACHE_E_SHAPE, "varlen_attn: unsupported configuration");
+  if (dtype == ACACHE_BF16) return launch_attn_any_head_dim<ACACHE_BF16>(p, mode, total_q, st);
+  return launch_attn_any_head_dim<ACACHE_F16>(p, mode, total_q, st);
 }

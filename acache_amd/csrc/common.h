@@ -70,10 +70,15 @@ __device__ __forceinline__ void store16_stream(void *p, const vec16 &v) {
 // Write-through streaming store (nt sc0 sc1): the line goes to memory without being kept in L2 or the
 // Infinity Cache.  For the relocation output, 9 GB written once per launch, this measured 2 % faster than
 // the plain non-temporal store.
+//
+// The s_nop behind the store is required: a VALU instruction must not overwrite the data registers of a
+// vector store of more than 8 bytes in the two issue slots after it (the store has not read them yet), and
+// the compiler's hazard pass does not see a store inside inline assembly; without it the register allocator
+// is free to reuse the first data registers for the next address computation right away.
 __device__ __forceinline__ void store16_writethrough(void *p, const vec16 &v) {
   typedef uint32_t u4 __attribute__((ext_vector_type(4)));
   const u4 t = {v.w[0], v.w[1], v.w[2], v.w[3]};
-  asm volatile("global_store_dwordx4 %0, %1, off nt sc0 sc1" ::"v"(p), "v"(t) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off nt sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(t) : "memory");
 }
 
 // ------------------------------------------------------- element <-> fp32 ----

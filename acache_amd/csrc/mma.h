@@ -36,11 +36,11 @@ template <> struct Mma<ACACHE_F16> {
 };
 
 // Rotate the (lo, hi) 16-byte chunk pair of one row: elements d0..d0+7 and
-// d0+D/2..d0+D/2+7.  sign = +1: x*cos + rot_half(x)*sin (key side);
+// d0+half..d0+half+7, half = head_dim / 2.  sign = +1: x*cos + rot_half(x)*sin (key side);
 // sign = -1: x*cos - rot_half(x)*sin (query side).  Rounded once to DTYPE.
-template <int DTYPE, int D>
-__device__ __forceinline__ void rotate_pair(vec16 &lo, vec16 &hi, const float *cos_row,
-                                            const float *sin_row, int d0, float sign) {
+template <int DTYPE>
+__device__ __forceinline__ void rotate_pair_half(vec16 &lo, vec16 &hi, const float *cos_row,
+                                                 const float *sin_row, int d0, int half, float sign) {
   // products and sum rounded separately, exactly like the stand-alone relocation
   // kernel, so key-side attention and attention over a materialised copy see
   // bit-identical keys
@@ -52,12 +52,18 @@ __device__ __forceinline__ void rotate_pair(vec16 &lo, vec16 &hi, const float *c
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     const float cl = cos_row[d0 + j], sl = sign * sin_row[d0 + j];
-    const float ch = cos_row[d0 + D / 2 + j], sh = sign * sin_row[d0 + D / 2 + j];
+    const float ch = cos_row[d0 + half + j], sh = sign * sin_row[d0 + half + j];
     ya[j] = a[j] * cl + (-b[j]) * sl;
     yb[j] = b[j] * ch + a[j] * sh;
   }
   lo = E::pack(ya);
   hi = E::pack(yb);
+}
+
+template <int DTYPE, int D>
+__device__ __forceinline__ void rotate_pair(vec16 &lo, vec16 &hi, const float *cos_row,
+                                            const float *sin_row, int d0, float sign) {
+  rotate_pair_half<DTYPE>(lo, hi, cos_row, sin_row, d0, D / 2, sign);
 }
 
 }  // namespace acache

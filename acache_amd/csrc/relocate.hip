@@ -36,6 +36,7 @@ struct RelocateParams {
   int32_t H_kv;
   int32_t rope_rows;
   int32_t const_delta;
+  int32_t D;  // head_dim (read by the any-head_dim kernel only)
 };
 
 template <int DTYPE, int D, int LPB>
@@ -137,6 +138,81 @@ __global__ __launch_bounds__(256) void relocate_kernel(RelocateParams p) {
   }
 }
 
+// Any other head_dim whose half row is a whole number of 16-byte chunks (bf16 / fp16: a multiple of 16,
+// fp32: a multiple of 8).  Same lane layout and the same arithmetic with the row geometry in registers
+// instead of template constants: one thread per (row, chunk pair), rows packed densely into blocks.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void relocate_any_kernel(RelocateParams p) {
+  using E = Elem<DTYPE>;
+  constexpr int VEC = E::kPerVec;
+  const int D = p.D;
+  const int half_bytes = D / 2 * E::kBytes;
+  const int lpr = half_bytes / 16;
+
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = g / lpr;
+  const int lane = (int)(g - row * lpr);
+  if (row >= p.T * p.H_kv) return;
+  const int64_t token = row / p.H_kv;
+  const int head = (int)(row - token * p.H_kv);
+
+  const int64_t slot = p.slot_map ? (int64_t)p.slot_map[token] : token;
+  const int32_t dlt = p.delta ? p.delta[token] : p.const_delta;
+  const int32_t adlt = dlt < 0 ? -dlt : dlt;
+  const bool rotate = dlt != 0;
+  const bool valid = slot >= 0 && slot < p.num_slots && (!rotate || adlt < p.rope_rows);
+
+  const int64_t row_bytes = (int64_t)D * E::kBytes;
+  const int64_t src_off = (slot * p.H_kv + head) * row_bytes + (int64_t)lane * 16;
+  const int64_t dst_off = (token * p.H_kv + head) * row_bytes + (int64_t)lane * 16;
+  const int64_t layer = blockIdx.y;
+
+  vec16 k_lo{{0, 0, 0, 0}}, k_hi = k_lo, v_lo = k_lo, v_hi = k_lo;
+  if (valid) {
+    const char *ks = p.k_cache + layer * p.cache_layer_bytes + src_off;
+    const char *vs = p.v_cache + layer * p.cache_layer_bytes + src_off;
+    k_lo = load16_stream(ks);
+    k_hi = load16_stream(ks + half_bytes);
+    v_lo = load16_stream(vs);
+    v_hi = load16_stream(vs + half_bytes);
+    if (rotate) {
+      const int d0 = lane * VEC;
+      const float *cr = p.cos_tab + (int64_t)adlt * D + d0;
+      const float *sr = p.sin_tab + (int64_t)adlt * D + d0;
+      const float sgn = dlt < 0 ? -1.0f : 1.0f;  // sin is odd, cos is even: rotate by -|d|
+      float a[VEC], b[VEC], ya[VEC], yb[VEC];
+      E::unpack(k_lo, a);
+      E::unpack(k_hi, b);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        const float cl = cr[j], sl = sgn * sr[j];
+        const float ch = cr[D / 2 + j], sh = sgn * sr[D / 2 + j];
+        ya[j] = a[j] * cl + (-b[j]) * sl;
+        yb[j] = b[j] * ch + a[j] * sh;
+      }
+      k_lo = E::pack(ya);
+      k_hi = E::pack(yb);
+    }
+  }
+  char *kd = p.out_k + layer * p.out_layer_bytes + dst_off;
+  char *vd = p.out_v + layer * p.out_layer_bytes + dst_off;
+  store16_writethrough(kd, k_lo);
+  store16_writethrough(kd + half_bytes, k_hi);
+  store16_writethrough(vd, v_lo);
+  store16_writethrough(vd + half_bytes, v_hi);
+}
+
+template <int DTYPE>
+static int launch_relocate_any(const RelocateParams &p, hipStream_t stream) {
+  const int lpr = p.D / 2 * Elem<DTYPE>::kBytes / 16;
+  const int64_t threads = p.T * p.H_kv * lpr;
+  if (threads == 0 || p.L == 0) return 0;
+  const int64_t gx = (threads + 255) / 256;
+  if (gx > 0x7fffffffLL || p.L > 65535) return fail(ACACHE_E_SHAPE, "relocate: grid too large");
+  hipLaunchKernelGGL((relocate_any_kernel<DTYPE>), dim3((unsigned)gx, (unsigned)p.L), dim3(256), 0, stream, p);
+  return launch_status("relocate_any_kernel");
+}
+
 template <int DTYPE, int D>
 static int launch_relocate(const RelocateParams &p, hipStream_t stream) {
   constexpr int LPR = D / 2 * Elem<DTYPE>::kBytes / 16;
@@ -165,8 +241,15 @@ static int dispatch_relocate(const RelocateParams &p, int dtype, int D, hipStrea
   ACACHE_CASE(ACACHE_F32, 128)
   ACACHE_CASE(ACACHE_F32, 64)
 #undef ACACHE_CASE
-  if (dtype_bytes(dtype) == 0) return fail(ACACHE_E_DTYPE, "relocate: unknown dtype %d", dtype);
-  return fail(ACACHE_E_SHAPE, "relocate: head_dim %d not supported (64 or 128)", D);
+  const int es = dtype_bytes(dtype);
+  if (es == 0) return fail(ACACHE_E_DTYPE, "relocate: unknown dtype %d", dtype);
+  if (D <= 0 || D > 1024 || (D / 2 * es) % 16 != 0 || D % 2 != 0)
+    return fail(ACACHE_E_SHAPE, "relocate: head_dim %d not supported (half a row must be a multiple of 16 bytes)", D);
+  RelocateParams q = p;
+  q.D = D;
+  if (dtype == ACACHE_BF16) return launch_relocate_any<ACACHE_BF16>(q, stream);
+  if (dtype == ACACHE_F16) return launch_relocate_any<ACACHE_F16>(q, stream);
+  return launch_relocate_any<ACACHE_F32>(q, stream);
 }
 
 }  // namespace acache
@@ -202,7 +285,7 @@ extern "C" int acache_relocate_rope_gather(
   p.slot_map = slot_map; p.delta = delta; p.cos_tab = rope_cos; p.sin_tab = rope_sin;
   p.T = T; p.num_slots = num_slots;
   p.cache_layer_bytes = cache_layer_stride * es; p.out_layer_bytes = out_layer_stride * es;
-  p.L = L; p.H_kv = H_kv; p.rope_rows = rope_rows; p.const_delta = 0;
+  p.L = L; p.H_kv = H_kv; p.rope_rows = rope_rows; p.const_delta = 0; p.D = D;
   return dispatch_relocate(p, dtype, D, (hipStream_t)stream);
 }
 
@@ -240,6 +323,6 @@ extern "C" int acache_materialize_relocated_affix(
   p.slot_map = nullptr; p.delta = nullptr; p.cos_tab = rope_cos; p.sin_tab = rope_sin;
   p.T = affix_len; p.num_slots = num_slots;
   p.cache_layer_bytes = cache_layer_stride * es; p.out_layer_bytes = cache_layer_stride * es;
-  p.L = L; p.H_kv = H_kv; p.rope_rows = rope_rows; p.const_delta = affix_shift;
+  p.L = L; p.H_kv = H_kv; p.rope_rows = rope_rows; p.const_delta = affix_shift; p.D = D;
   return dispatch_relocate(p, dtype, D, (hipStream_t)stream);
 }

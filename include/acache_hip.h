@@ -70,6 +70,8 @@ const char *acache_last_error(void);
  * or whose |delta| >= rope_rows is written as zeros (K and V).
  *
  * rope_cos / rope_sin: fp32 [rope_rows, D] contiguous, may be NULL iff delta is NULL.
+ * D: half a row must be a whole number of 16-byte chunks (bf16 / f16: a multiple of 16,
+ * f32: a multiple of 8); 128 and 64 take the tuned kernel.
  * cache_layer_stride / out_layer_stride: elements between consecutive layers.
  * Token rows are contiguous: [.., H_kv, D] with strides (H_kv*D, D, 1).
  */
@@ -304,8 +306,10 @@ int acache_build_slot_layout(
  * as zeros instead of being left uninitialised, and no host synchronisation is
  * needed: the grid is sized from total_q and B.
  *
- * Supported: D == 128 or 64, dtype bf16 or f16, H % H_kv == 0, scale > 0 (ACACHE_E_RANGE
- * otherwise).  A key whose slot lies outside [0, num_slots) reads as a zero row.
+ * Supported: D a multiple of 16 up to 256 (128 and 64 take the tuned kernels, every other
+ * width a padded one, as the reference pads to the next power of two, lines 517-522),
+ * dtype bf16 or f16, H % H_kv == 0, scale > 0 (ACACHE_E_RANGE otherwise).  A key whose
+ * slot lies outside [0, num_slots) reads as a zero row.
  * q / out: [total_q, H, D] with given token and head strides (innermost 1).
  * k_cache / v_cache: [num_slots, H_kv, D] with given slot and head strides.
  */

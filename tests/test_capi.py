@@ -44,8 +44,8 @@ def test_argument_errors_are_reported_without_a_device():
     # shift beyond the table
     rc = lib.acache_materialize_relocated_affix(p, p, p, p, 8, 4, 16, 1, 2, 64, 0, 32, 16, 0, None)
     assert rc == -4
-    # unsupported head_dim
-    rc = lib.acache_materialize_relocated_affix(p, p, p, p, 8, 4, 1, 1, 2, 96, 0, 32, 16, 0, None)
+    # unsupported head_dim: half a bf16 row of 100 elements is not a whole number of 16-byte chunks
+    rc = lib.acache_materialize_relocated_affix(p, p, p, p, 8, 4, 1, 1, 2, 100, 0, 32, 16, 0, None)
     assert rc == -3
     # NULL payload
     rc = lib.acache_relocate_rope_gather(None, p, p, p, p, None, None, None, 4, 1, 2, 64, 0, 32, 0, 0, 0, None)

@@ -140,6 +140,85 @@ def test_key_side_equals_materialised_bitwise_reference_geometry(device):
     assert torch.equal(materialised, key_side)
 
 
+def test_large_head_dim_matches_dense_reference(device):
+    """tests/test_attention_kernels.py:237-291: head_dim 160 (not a power of two), fp16, 8 blocks of 8, H=4, Hkv=2,
+    q=[3,2], kv=[7,5], random slot maps; tolerance 5e-2 there."""
+    torch.manual_seed(0)
+    H, Hkv, D = 4, 2, 160
+    q = torch.randn(5, H, D).to(torch.float16)
+    kc = torch.randn(8, 8, Hkv, D).to(torch.float16)
+    vc = torch.randn_like(kc)
+    maps = torch.cat([torch.randperm(64)[:7], torch.randperm(64)[:5]]).to(torch.int32)
+    cu_q = torch.tensor([0, 3, 5], dtype=torch.int32)
+    cu_k = torch.tensor([0, 7, 12], dtype=torch.int32)
+    want = torch.cat([O.dense_attention_reference(q[a:b], kc.view(-1, Hkv, D)[maps[c:d].long()],
+                                                  vc.view(-1, Hkv, D)[maps[c:d].long()], H, Hkv)
+                      for (a, b), (c, d) in (((0, 3), (0, 7)), ((3, 5), (7, 12)))])
+    got = ops.acache_attention(q.to(device), kc.to(device), vc.to(device), cu_q.to(device), cu_k.to(device),
+                               maps.to(device))
+    _close(got, want)
+
+
+@pytest.mark.parametrize("D", [16, 32, 96, 160, 192, 256])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_other_head_dims_all_relocation_modes(device, D, dtype):
+    """Every width that is a multiple of 16 up to 256 runs on the padded kernel: plain ragged batch, then an infix
+    affix relocated on the key side and on the query side against the oracle, and key side == plain attention over
+    the materialised copy, bit for bit."""
+    g = torch.Generator().manual_seed(D)
+    H, Hkv, S = 6, 2, 512
+    q_lens = [1, 17, 0, 70, 64, 33]
+    kv_lens = [1, 63, 40, 130, 0, 64]
+    q = (torch.randn(sum(q_lens), H, D, generator=g) / D ** 0.25).to(dtype)
+    kc = (torch.randn(S, Hkv, D, generator=g) / D ** 0.25).to(dtype)
+    vc = torch.randn(S, Hkv, D, generator=g).to(dtype)
+    slots = torch.cat([torch.randperm(S, generator=g)[:n] for n in kv_lens]).to(torch.int32)
+    cu_q = torch.tensor([0] + torch.tensor(q_lens).cumsum(0).tolist(), dtype=torch.int32)
+    cu_k = torch.tensor([0] + torch.tensor(kv_lens).cumsum(0).tolist(), dtype=torch.int32)
+    dev = lambda t: None if t is None else t.to(device)
+    want = O.acache_attention(q, kc, vc, cu_q, cu_k, slots)
+    got = ops.acache_attention(dev(q), dev(kc.view(S // 16, 16, Hkv, D)), dev(vc.view(S // 16, 16, Hkv, D)),
+                               dev(cu_q), dev(cu_k), dev(slots))
+    _close(got, want)
+    assert torch.all(got[cu_q[4]:cu_q[5]] == 0)            # the request without keys
+
+    # infix affix: A shared rows cached at positions 0..A-1, read at a0..a0+A-1, every fifth one an anchor
+    A, a0, tail, nq = 90, 37, 50, 45
+    cos, sin = O.rope_table(256, D, 1e4)
+    anchors = set(range(a0 + 2, a0 + A, 5))
+    read, nxt = [], 128
+    for pos in range(a0 + A + tail):
+        if a0 <= pos < a0 + A and pos not in anchors:
+            read.append(pos - a0)
+        else:
+            read.append(nxt)
+            nxt += 1
+    q1 = (torch.randn(nq, H, D, generator=g) / D ** 0.25).to(dtype)
+    cu_q1 = torch.tensor([0, nq], dtype=torch.int32)
+    cu_k1 = torch.tensor([0, len(read)], dtype=torch.int32)
+    shifts = torch.tensor([a0], dtype=torch.int32)
+    kc4, vc4 = dev(kc.view(S // 16, 16, Hkv, D)), dev(vc.view(S // 16, 16, Hkv, D))
+    want = O.acache_attention(q1, kc, vc, cu_q1, cu_k1, torch.tensor(read, dtype=torch.int32), shared_prefix_len=A,
+                              affix_shifts=shifts, rope_cos=cos, rope_sin=sin)
+    key_side = ops.acache_attention(dev(q1), kc4, vc4, dev(cu_q1), dev(cu_k1),
+                                    dev(torch.tensor(read, dtype=torch.int32)), shared_prefix_len=A,
+                                    affix_shifts=dev(shifts), rope_cos=dev(cos), rope_sin=dev(sin))
+    _close(key_side, want)
+    packed, n_shared = O.attention_read_layout(read, 0, A, a0, True)
+    query_side = ops.acache_attention(dev(q1), kc4, vc4, dev(cu_q1), dev(cu_k1),
+                                      dev(torch.tensor(packed, dtype=torch.int32)), shared_prefix_len=A,
+                                      shared_kv_lens=dev(torch.tensor([n_shared], dtype=torch.int32)),
+                                      affix_shifts=dev(shifts), rope_cos=dev(cos), rope_sin=dev(sin))
+    _close(query_side, want)
+    # materialise the affix at slots 300.., then plain attention over the copy
+    kl, vl = dev(kc)[None].clone(), dev(vc)[None].clone()
+    ops.materialize_relocated_affix(kl, vl, dev(cos), dev(sin), 300, A, a0)
+    mread = [300 + s if s < A else s for s in read]
+    materialised = ops.acache_attention(dev(q1), kl[0].view(S // 16, 16, Hkv, D), vl[0].view(S // 16, 16, Hkv, D),
+                                        dev(cu_q1), dev(cu_k1), dev(torch.tensor(mread, dtype=torch.int32)))
+    assert torch.equal(materialised, key_side)
+
+
 def test_query_side_relocation_reference_geometry(device):
     """tests/test_attention_kernels.py:294-368: keys cached post-RoPE at source positions, shared keys packed
     first, result compared with dense attention over keys rotated at their logical positions (fp16, tol 5e-2 there)."""

@@ -52,6 +52,38 @@ def test_relocate_gather_small_bit_exact(device, dtype, H, D):
     assert torch.equal(_bits(gv.cpu()), _bits(ev))
 
 
+@pytest.mark.parametrize("dtype,H,D", [(torch.bfloat16, 2, 160), (torch.float16, 5, 96), (torch.float32, 3, 40),
+                                       (torch.bfloat16, 1, 16), (torch.bfloat16, 4, 256), (torch.float32, 2, 72)])
+def test_relocate_gather_other_head_dims_bit_exact(device, dtype, H, D):
+    """Head dims other than 64 / 128 (the reference takes any width: acache_attention.py:100-101) go through the
+    kernel with the row geometry in registers; same lane layout, same arithmetic, same bits.  Also the in-place
+    materialise form and out-of-range rows."""
+    torch.manual_seed(D)
+    L, S, T = 2, 90, 77
+    cos, sin = O.rope_table(128, D, 1e4)
+    k = torch.randn(L, S, H, D).to(dtype)
+    v = torch.randn(L, S, H, D).to(dtype)
+    slot = torch.randint(0, S, (T,), dtype=torch.int32)
+    delta = torch.randint(-127, 128, (T,), dtype=torch.int32)
+    delta[::5] = 0
+    ek, ev = O.relocate_rope_gather(k, v, slot, delta, cos, sin)
+    gk, gv = ops.relocate_rope_gather(k.to(device), v.to(device), slot.to(device), delta.to(device),
+                                      cos.to(device), sin.to(device))
+    assert torch.equal(_bits(gk.cpu()), _bits(ek))
+    assert torch.equal(_bits(gv.cpu()), _bits(ev))
+    bad = slot.clone()
+    bad[1], bad[2] = -1, S
+    gk, gv = ops.relocate_rope_gather(k.to(device), v.to(device), bad.to(device), delta.to(device),
+                                      cos.to(device), sin.to(device))
+    assert torch.all(gk[:, 1:3] == 0) and torch.all(gv[:, 1:3] == 0)
+    assert torch.equal(_bits(gk[:, 3:].cpu()), _bits(ek[:, 3:]))
+    mk, mv = k.clone(), v.clone()
+    O.materialize_relocated_affix(mk, mv, cos, sin, 40, 33, 21)
+    dk, dv = k.to(device), v.to(device)
+    ops.materialize_relocated_affix(dk, dv, cos.to(device), sin.to(device), 40, 33, 21)
+    assert torch.equal(_bits(dk.cpu()), _bits(mk)) and torch.equal(_bits(dv.cpu()), _bits(mv))
+
+
 def test_pure_gather_and_out_of_range_rows(device):
     torch.manual_seed(2)
     L, S, H, D, T = 2, 64, 4, 128, 40
