@@ -39,3 +39,7 @@ class Config:
     # not in the reference: replay the block-refinement forward from a captured HIP graph (same kernels, same
     # results, no per-launch host cost); re-captured whenever the attention metadata of the step changes
     decode_hip_graph: bool = False
+    # not in the reference (which probes one request per forward, model_runner.py:873): requests per
+    # anchor-selection probe forward; 0 = all newly admitted requests at once.  Selection is the same either way
+    # (the importance kernels are deterministic and requests do not interact).
+    anchor_selection_batch_size: int = 1

@@ -493,9 +493,13 @@ class ModelRunner:
 
     def _select_anchor_positions_for_sequences(self, seqs, prefix_token_ids, allow_kv_cache_resize,
                                                minimum_blocks=None):
-        # one request per probe forward, as the reference does (model_runner.py:873)
-        for seq in seqs:
-            seq.set_anchor_positions(self._compute_anchor_positions_batch([seq])[0])
+        # one request per probe forward by default, as the reference does (model_runner.py:873);
+        # Config.anchor_selection_batch_size widens the probe (0: all admitted requests in one forward)
+        step = int(getattr(self.config, "anchor_selection_batch_size", 1) or 0) or len(seqs)
+        for i in range(0, len(seqs), step):
+            batch = seqs[i:i + step]
+            for seq, anchors in zip(batch, self._compute_anchor_positions_batch(batch)):
+                seq.set_anchor_positions(anchors)
 
     def _prepare_admitted_sequences_for_acache(self, seqs, prefix_token_ids, allow_kv_cache_resize):
         if not seqs:

@@ -326,7 +326,8 @@ def engine_bench(torch, device, args):
         return Config(hf_config=cfg, mask_id=cfg.mask_token_id, recompute_batch_size=4, max_num_seqs=0,
                       gen_length=gen, block_length=block, threshold=0.9, cache_block_size=256,
                       num_kvcache_blocks=args.engine_kv_blocks, temperature=0.0, enable_acache=enable,
-                      anchor_ratio=ratio, profile_timing=True, decode_hip_graph=args.engine_graph)
+                      anchor_ratio=ratio, profile_timing=True, decode_hip_graph=args.engine_graph,
+                      anchor_selection_batch_size=args.engine_probe_batch)
 
     def prompts_of(gen_length):
         nonlocal gen
@@ -390,6 +391,8 @@ def main():
     ap.add_argument("--engine", action="store_true", help="run the engine-step sweep (configs[4]) instead")
     ap.add_argument("--engine-graph", action="store_true",
                     help="replay the refinement forward from a captured HIP graph (measured: no gain, the loop is GPU-bound)")
+    ap.add_argument("--engine-probe-batch", type=int, default=0,
+                    help="requests per anchor-selection probe forward (0 = all admitted requests at once, 1 = the reference's choice)")
     ap.add_argument("--engine-layers", type=int, default=32)
     ap.add_argument("--engine-batch", type=int, default=16)
     ap.add_argument("--engine-affix", type=int, default=1000)

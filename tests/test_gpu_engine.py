@@ -232,3 +232,37 @@ def test_hip_graph_replay_of_refinement_steps_gives_the_same_tokens(device, use_
         replayed, nfe_graph, timing = run(True)
         assert replayed == eager and nfe_graph == nfe_eager
         assert all(63 not in g for g in replayed)
+
+
+@pytest.mark.parametrize("placement", ["prefix", "infix"])
+def test_batched_probe_at_admission_selects_the_same_anchors(device, placement):
+    """Config.anchor_selection_batch_size = 0 probes all admitted requests in one forward instead of one forward
+    per request (the reference's choice, model_runner.py:873): same anchors, same generated tokens."""
+    cfg, model = _model(device, seed=3)
+    affix = list(range(20, 32))
+
+    def make(i):
+        if placement == "prefix":
+            return Sequence(affix + [40 + i, 41 + i, 42 + i][: 2 + i % 2], gen_length=4, block_length=4,
+                            cache_block_size=8, mask_id=63, prompt_affix_len=len(affix))
+        return Sequence([2 + i] * (1 + i % 3) + affix + [40 + i], gen_length=4, block_length=4, cache_block_size=8,
+                        mask_id=63, prompt_affix_start=1 + i % 3, prompt_affix_end=1 + i % 3 + len(affix))
+
+    results = []
+    for probe_batch in (1, 0, 3):
+        runner = ModelRunner(model, _serve(cfg, recompute_batch_size=2, max_num_seqs=0, num_kvcache_blocks=40,
+                                           anchor_ratio=0.4, anchor_selection_batch_size=probe_batch))
+        calls = []
+        real = runner._compute_anchor_positions_batch
+
+        def spy(batch, real=real, calls=calls):
+            calls.append(len(batch))
+            return real(batch)
+
+        runner._compute_anchor_positions_batch = spy
+        seqs = [make(i) for i in range(5)]
+        out, _ = runner.generate_with_acache(seqs)
+        results.append(([list(s.anchor_positions) for s in seqs], out))
+        assert calls == {1: [1] * 5, 0: [5], 3: [3, 2]}[probe_batch]
+    assert results[0] == results[1] == results[2]
+    assert all(len(a) == 5 for a in results[0][0])          # ceil(0.4 * 12) anchors per request
