@@ -46,45 +46,41 @@ struct ImportanceParams {
   int32_t H_kv;
   int32_t rope_rows;
   int32_t max_row_tiles;
+  int32_t D;  // head_dim
 };
 
-// Operand fragments of 16 rows x D: lane (li, lg) takes row `row_ptr` (NULL: zeros), elements
-// 32*ks + 8*lg .. + 8, optionally rotated by the table row (cr, sr).
-template <int DTYPE, int D>
-__device__ __forceinline__ void load_rows(vec16 (&f)[D / 32], const char *row_ptr, int lg, const float *cr,
-                                          const float *sr) {
-  constexpr int KS = D / 32;
+// Operand fragments of 16 rows x head_dim, KS slabs of 32 elements: lane (li, lg) takes row `row_ptr`
+// (NULL: zeros), elements 32*ks + 8*lg .. + 8; chunks at or past head_dim (a multiple of 16) read as zeros.
+template <int KS>
+__device__ __forceinline__ void load_rows(vec16 (&f)[KS], const char *row_ptr, int lg, int head_dim) {
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
-    f[ks] = row_ptr ? load16(row_ptr + (32 * ks + 8 * lg) * 2) : vec16{{0, 0, 0, 0}};
-  if (row_ptr && cr) {
-#pragma unroll
-    for (int ks = 0; ks < KS / 2; ++ks) rotate_pair<DTYPE, D>(f[ks], f[ks + KS / 2], cr, sr, 32 * ks + 8 * lg, 1.0f);
-  }
+    f[ks] = row_ptr && 32 * ks + 8 * lg < head_dim ? load16(row_ptr + (32 * ks + 8 * lg) * 2) : vec16{{0, 0, 0, 0}};
 }
 
 // Re-rotate the cached affix keys once per request: k_rot[b, a, h, :] = rot(K[affix_slot0 + a, h, :], shift_b).
 // One row of D elements per LPR lanes, the rotate-half partner in the same lane; fp32 products and sum rounded
 // separately, one rounding to the cache type (the arithmetic of the relocation kernel).
-template <int DTYPE, int D>
+template <int DTYPE>
 __global__ __launch_bounds__(256) void importance_rotate_kernel(ImportanceParams p) {
 #pragma clang fp contract(off)
   using E = Elem<DTYPE>;
   constexpr int VEC = E::kPerVec;
-  constexpr int HALF_BYTES = D * E::kBytes / 2;
-  constexpr int LPR = HALF_BYTES / 16;
-  constexpr int RPB = 256 / LPR;
+  const int D = p.D;
+  const int half_bytes = D * E::kBytes / 2;
+  const int lpr = half_bytes / 16;
   const int b = blockIdx.y;
-  const int lane = threadIdx.x % LPR;
-  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = g / lpr;
+  const int lane = (int)(g - row * lpr);
   if (row >= (int64_t)p.A * p.H_kv) return;
   const int64_t a = row / p.H_kv;
   const int head = (int)(row - a * p.H_kv);
   int shift = p.shifts[b];
   if (shift < 0 || shift >= p.rope_rows) shift = 0;
   const char *src = p.k_cache + (p.affix_slot0 + a) * p.kv_slot_bytes + (int64_t)head * p.kv_head_bytes + lane * 16;
-  char *dst = p.k_rot + (int64_t)b * p.k_rot_bytes + row * (2 * HALF_BYTES) + lane * 16;
-  vec16 lo = load16(src), hi = load16(src + HALF_BYTES);
+  char *dst = p.k_rot + (int64_t)b * p.k_rot_bytes + row * (2 * half_bytes) + lane * 16;
+  vec16 lo = load16(src), hi = load16(src + half_bytes);
   if (shift != 0) {
     const float *cr = p.cos_tab + (int64_t)shift * D + lane * VEC;
     const float *sr = p.sin_tab + (int64_t)shift * D + lane * VEC;
@@ -100,17 +96,17 @@ __global__ __launch_bounds__(256) void importance_rotate_kernel(ImportanceParams
     hi = E::pack(ya);
   }
   store16(dst, lo);
-  store16(dst + HALF_BYTES, hi);
+  store16(dst + half_bytes, hi);
 }
 
 constexpr int kKeysPerStep = 64;  // keys a wave scores per loop step (four independent 16-key tiles in flight)
 
 constexpr int kRowTilesPerWave = 4;  // 16-row tiles of mask queries a stats wave owns (keys are loaded once for all)
 
-template <int DTYPE, int D>
+template <int DTYPE, int KS>
 __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams p) {
-  constexpr int KS = D / 32;
   constexpr int NQ = kRowTilesPerWave;
+  const int D = p.D;  // KS = ceil(D / 32) slabs; the last one may be half empty
   using M = Mma<DTYPE>;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
@@ -127,8 +123,8 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
     const int r = row0 + 16 * qt + li;
-    load_rows<DTYPE, D>(qf[qt], r < n_rows ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
-                                           : nullptr, lg, nullptr, nullptr);
+    load_rows<KS>(qf[qt], r < n_rows ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
+                                     : nullptr, lg, D);
   }
   const int64_t slot_bytes = p.k_rot ? (int64_t)p.H_kv * D * 2 : p.kv_slot_bytes;
   const char *k_base = p.k_rot ? p.k_rot + (int64_t)b * p.k_rot_bytes + (int64_t)kvh * D * 2
@@ -143,7 +139,7 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       const int a = a0 + 16 * nt + li;
-      load_rows<DTYPE, D>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, nullptr, nullptr);
+      load_rows<KS>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, D);
     }
 #pragma unroll
     for (int qt = 0; qt < NQ; ++qt) {
@@ -184,10 +180,10 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
 
 // One wave per (request, head, 64 affix keys): the keys stay in registers, the request's mask rows stream by.
 // The wave is the only writer of partial[b, h, a0 .. a0 + 64).
-template <int DTYPE, int D>
+template <int DTYPE, int KS>
 __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams p) {
-  constexpr int KS = D / 32;
   using M = Mma<DTYPE>;
+  const int D = p.D;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
   const int b = blockIdx.z;
@@ -206,14 +202,14 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
     const int a = a0 + 16 * nt + li;
-    load_rows<DTYPE, D>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, nullptr, nullptr);
+    load_rows<KS>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, D);
   }
   float col[4][4] = {};
   auto fetch = [&](int r0, vec16 (&qf)[KS], float2 &st) __attribute__((always_inline)) {
     const int r = r0 + li;
     const bool live = r < n_rows;
-    load_rows<DTYPE, D>(qf, live ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
-                                 : nullptr, lg, nullptr, nullptr);
+    load_rows<KS>(qf, live ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
+                           : nullptr, lg, D);
     st = live ? p.stats[(int64_t)(m0 + r) * p.H + h] : make_float2(0.0f, INFINITY);  // 1 / inf = 0: adds nothing
   };
   vec16 q_cur[KS], q_next[KS];
@@ -291,7 +287,8 @@ extern "C" int acache_affix_importance(
     void *stream) {
   if (dtype != ACACHE_BF16 && dtype != ACACHE_F16)
     return fail(ACACHE_E_DTYPE, "affix_importance: dtype %d not supported (bf16 or f16)", dtype);
-  if (D != 128 && D != 64) return fail(ACACHE_E_SHAPE, "affix_importance: head_dim %d not supported (64 or 128)", D);
+  if (D < 16 || D > 256 || D % 16 != 0)
+    return fail(ACACHE_E_SHAPE, "affix_importance: head_dim %d not supported (a multiple of 16 up to 256)", D);
   if (B < 0 || affix_len < 0 || total_mask_rows < 0 || max_mask_rows < 0 || H <= 0 || H_kv <= 0 || H % H_kv)
     return fail(ACACHE_E_SHAPE, "affix_importance: bad sizes (B %d, A %d, H %d, H_kv %d)", B, affix_len, H, H_kv);
   if (B == 0 || affix_len == 0 || total_mask_rows == 0 || max_mask_rows == 0) return 0;
@@ -323,35 +320,38 @@ extern "C" int acache_affix_importance(
   p.kv_slot_bytes = kv_slot_stride * 2; p.kv_head_bytes = kv_head_stride * 2;
   p.affix_slot0 = affix_slot0;
   p.scale_log2e = scale * 1.4426950408889634f;
-  p.A = affix_len; p.B = B; p.H = H; p.H_kv = H_kv; p.rope_rows = rope_rows;
+  p.A = affix_len; p.B = B; p.H = H; p.H_kv = H_kv; p.rope_rows = rope_rows; p.D = D;
   p.max_row_tiles = (max_mask_rows + 15) / 16;
   hipStream_t s = (hipStream_t)stream;
-  const int rows_per_block = 256 / (D * 2 / 32);
-  const dim3 grid0((unsigned)(((int64_t)affix_len * H_kv + rows_per_block - 1) / rows_per_block), (unsigned)B);
+  const int lanes_per_row = D * 2 / 32;
+  const dim3 grid0((unsigned)(((int64_t)affix_len * H_kv * lanes_per_row + 255) / 256), (unsigned)B);
   const int row_groups = (p.max_row_tiles + kRowTilesPerWave - 1) / kRowTilesPerWave;
   const dim3 grid1((unsigned)((int64_t)B * row_groups), (unsigned)((H + 3) / 4));
   const dim3 grid2((unsigned)((affix_len + kKeysPerStep - 1) / kKeysPerStep), (unsigned)((H + 3) / 4), (unsigned)B);
   const dim3 grid3((unsigned)((affix_len + 255) / 256), (unsigned)B);
-#define ACACHE_CASE(DT, DD)                                                                       \
-  if (dtype == DT && D == DD) {                                                                   \
+  const int slabs = (D + 31) / 32;
+#define ACACHE_CASE(DT, SLABS)                                                                    \
+  if (dtype == DT && slabs == SLABS) {                                                            \
     if (p.k_rot) {                                                                                \
-      hipLaunchKernelGGL((importance_rotate_kernel<DT, DD>), grid0, dim3(256), 0, s, p);          \
+      hipLaunchKernelGGL((importance_rotate_kernel<DT>), grid0, dim3(256), 0, s, p);              \
       const int rc0 = launch_status("importance_rotate_kernel");                                  \
       if (rc0) return rc0;                                                                        \
     }                                                                                             \
-    hipLaunchKernelGGL((importance_stats_kernel<DT, DD>), grid1, dim3(256), 0, s, p);             \
+    hipLaunchKernelGGL((importance_stats_kernel<DT, SLABS>), grid1, dim3(256), 0, s, p);          \
     const int rc = launch_status("importance_stats_kernel");                                      \
     if (rc) return rc;                                                                            \
-    hipLaunchKernelGGL((importance_colsum_kernel<DT, DD>), grid2, dim3(256), 0, s, p);            \
+    hipLaunchKernelGGL((importance_colsum_kernel<DT, SLABS>), grid2, dim3(256), 0, s, p);         \
     const int rc2 = launch_status("importance_colsum_kernel");                                    \
     if (rc2) return rc2;                                                                          \
     hipLaunchKernelGGL(importance_reduce_kernel, grid3, dim3(256), 0, s, p);                      \
     return launch_status("importance_reduce_kernel");                                             \
   }
-  ACACHE_CASE(ACACHE_BF16, 128)
-  ACACHE_CASE(ACACHE_BF16, 64)
-  ACACHE_CASE(ACACHE_F16, 128)
-  ACACHE_CASE(ACACHE_F16, 64)
+#define ACACHE_SLABS(DT) \
+  ACACHE_CASE(DT, 4) ACACHE_CASE(DT, 2) ACACHE_CASE(DT, 1) ACACHE_CASE(DT, 3) \
+  ACACHE_CASE(DT, 5) ACACHE_CASE(DT, 6) ACACHE_CASE(DT, 7) ACACHE_CASE(DT, 8)
+  ACACHE_SLABS(ACACHE_BF16)
+  ACACHE_SLABS(ACACHE_F16)
+#undef ACACHE_SLABS
 #undef ACACHE_CASE
   return fail(ACACHE_E_SHAPE, "affix_importance: unsupported dtype / head_dim");
 }

@@ -32,6 +32,7 @@ struct RopeScatterParams {
   int32_t H;
   int32_t H_kv;
   int32_t rope_rows;
+  int32_t D;  // head_dim (read by the any-head_dim kernel only)
 };
 
 template <int DTYPE, int D>
@@ -107,6 +108,63 @@ __global__ __launch_bounds__(256) void rope_scatter_kernel(RopeScatterParams p) 
   }
 }
 
+// Any other head_dim whose half row is a whole number of 16-byte chunks: the same lane layout and
+// arithmetic with the row geometry in registers; a lane re-reads its table entries for every row it visits.
+template <int DTYPE>
+__global__ __launch_bounds__(256) void rope_scatter_any_kernel(RopeScatterParams p) {
+  using E = Elem<DTYPE>;
+  constexpr int VEC = E::kPerVec;
+  const int D = p.D;
+  const int row_bytes = D * E::kBytes;
+  const int half_bytes = row_bytes / 2;
+  const int lpr = half_bytes / 16;   // lanes per rotated row
+  const int ch = row_bytes / 16;     // chunks per copied row
+
+  const int64_t token = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t pos = p.positions[token];
+  const bool rotate = pos >= 0 && pos < p.rope_rows;
+  int64_t slot = p.slot_map ? (int64_t)p.slot_map[token] : -1;
+  if (slot >= p.num_slots) slot = -1;
+
+  const int rows = p.H + p.H_kv;
+  for (int idx = tid; idx < rows * lpr; idx += 256) {
+    const int row = idx / lpr, lane = idx - row * lpr;
+    const bool is_q = row < p.H;
+    const int head = is_q ? row : row - p.H;
+    char *src = is_q ? p.q + token * p.q_token_bytes : p.k + token * p.k_token_bytes;
+    src += (int64_t)head * row_bytes + lane * 16;
+    vec16 lo = load16(src), hi = load16(src + half_bytes);
+    if (rotate) {
+      const float *cr = p.cos_tab + pos * D + lane * VEC;
+      const float *sr = p.sin_tab + pos * D + lane * VEC;
+      float a[VEC], b[VEC], ya[VEC], yb[VEC];
+      E::unpack(lo, a);
+      E::unpack(hi, b);
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        ya[j] = a[j] * cr[j] + (-b[j]) * sr[j];
+        yb[j] = b[j] * cr[D / 2 + j] + a[j] * sr[D / 2 + j];
+      }
+      lo = E::pack(ya);
+      hi = E::pack(yb);
+      store16(src, lo);
+      store16(src + half_bytes, hi);
+    }
+    if (!is_q && slot >= 0) {
+      char *dst = p.k_cache + (slot * p.H_kv + head) * (int64_t)row_bytes + lane * 16;
+      store16(dst, lo);
+      store16(dst + half_bytes, hi);
+    }
+  }
+
+  if (slot >= 0) {
+    const char *vsrc = p.v + token * p.v_token_bytes;
+    char *vdst = p.v_cache + slot * p.H_kv * (int64_t)row_bytes;
+    for (int c = tid; c < p.H_kv * ch; c += 256) store16(vdst + (int64_t)c * 16, load16(vsrc + (int64_t)c * 16));
+  }
+}
+
 template <int DTYPE, int D>
 static int launch_rope_scatter(const RopeScatterParams &p, hipStream_t stream) {
   if (p.N > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "rope_qk_scatter: too many tokens (%lld)", (long long)p.N);
@@ -144,7 +202,7 @@ extern "C" int acache_rope_qk_scatter(
   p.positions = positions; p.slot_map = slot_map; p.cos_tab = rope_cos; p.sin_tab = rope_sin;
   p.N = N; p.num_slots = num_slots;
   p.q_token_bytes = q_token_stride * es; p.k_token_bytes = k_token_stride * es; p.v_token_bytes = v_token_stride * es;
-  p.H = H; p.H_kv = H_kv; p.rope_rows = rope_rows;
+  p.H = H; p.H_kv = H_kv; p.rope_rows = rope_rows; p.D = D;
   hipStream_t s = (hipStream_t)stream;
 #define ACACHE_CASE(DT, DD) \
   if (dtype == DT && D == DD) return launch_rope_scatter<DT, DD>(p, s);
@@ -155,5 +213,12 @@ extern "C" int acache_rope_qk_scatter(
   ACACHE_CASE(ACACHE_F32, 128)
   ACACHE_CASE(ACACHE_F32, 64)
 #undef ACACHE_CASE
-  return fail(ACACHE_E_SHAPE, "rope_qk_scatter: head_dim %d not supported (64 or 128)", D);
+  if (D <= 0 || D > 1024 || D % 2 != 0 || (D / 2 * es) % 16 != 0)
+    return fail(ACACHE_E_SHAPE, "rope_qk_scatter: head_dim %d not supported (half a row must be a multiple of 16 bytes)", D);
+  if (N > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "rope_qk_scatter: too many tokens (%lld)", (long long)N);
+  p.D = D;
+  if (dtype == ACACHE_BF16) hipLaunchKernelGGL((rope_scatter_any_kernel<ACACHE_BF16>), dim3((unsigned)N), dim3(256), 0, s, p);
+  else if (dtype == ACACHE_F16) hipLaunchKernelGGL((rope_scatter_any_kernel<ACACHE_F16>), dim3((unsigned)N), dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((rope_scatter_any_kernel<ACACHE_F32>), dim3((unsigned)N), dim3(256), 0, s, p);
+  return launch_status("rope_scatter_any_kernel");
 }

@@ -154,6 +154,7 @@ int acache_kv_scatter(
  * outside [0, num_slots) is skipped like -1; a position outside [0, rope_rows)
  * leaves the row unrotated.  q / k / v: [N, heads, D] with the given token
  * strides (heads contiguous, so the three may be views of one fused projection).
+ * D: half a row must be a whole number of 16-byte chunks (128 and 64 take the tuned kernel).
  */
 int acache_rope_qk_scatter(
     void *q, void *k, const void *v, void *k_cache, void *v_cache,
@@ -184,7 +185,8 @@ int acache_rope_qk_scatter(
  * device scratch of at least acache_affix_importance_workspace_bytes(total_mask_rows, B, H,
  * H_kv, D, affix_len, relocated = affix_shifts != NULL) bytes (row statistics, per-head
  * partial sums and, with relocation, one re-rotated copy of the affix keys per request,
- * passed between the launches), 16-byte aligned, owned by the caller.  max_mask_rows: an upper bound on the mask rows of one request.
+ * passed between the launches), 16-byte aligned, owned by the caller.  max_mask_rows: an upper bound on
+ * the mask rows of one request.  D: a multiple of 16 up to 256; dtype bf16 or f16.
  */
 int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_rows, int32_t B, int32_t H, int32_t H_kv,
                                                 int32_t D, int32_t affix_len, int32_t relocated);

@@ -4,7 +4,7 @@ Mirrors the invariants of the reference's engine tests
 (nano-vdllm/tests/test_model_runner_acache.py:305-430, 470-590, 605-687): shared-affix
 precompute state, batched == single anchor selection, ratio-1.0 ACache logits equal
 full-recompute logits for prefix / infix / suffix placement (tolerance 5e-2 there and here),
-and end-to-end generation for mixed layouts.  Head dim is 64 (the kernels support 64 and 128).
+and end-to-end generation for mixed layouts.  Head dim is 64 unless a test says otherwise.
 """
 import pytest
 import torch
@@ -17,9 +17,9 @@ from acache_amd.utils import reset_context
 pytestmark = pytest.mark.gpu
 
 
-def _model(device, seed=0, layers=2):
+def _model(device, seed=0, layers=2, d_model=256):
     torch.manual_seed(seed)
-    cfg = LLaDAConfig(vocab_size=64, d_model=256, n_heads=4, n_layers=layers, mlp_hidden_size=128,
+    cfg = LLaDAConfig(vocab_size=64, d_model=d_model, n_heads=4, n_layers=layers, mlp_hidden_size=128,
                       max_sequence_length=64, mask_token_id=63, rope_theta=10000.0)
     model = LLaDAModelLM(cfg, init_std=0.08).to(device=device, dtype=torch.bfloat16).eval()
     return cfg, model
@@ -83,11 +83,13 @@ def test_batched_anchor_selection_matches_single_sequence_selection(device):
     ],
 )
 @pytest.mark.parametrize("max_num_seqs", [4, 1])
+@pytest.mark.parametrize("d_model", [256, 64, 384])
 def test_full_recomputation_matches_baseline_for_all_affix_layouts(device, tokens, affix_start, affix_end,
-                                                                   generation_start, max_num_seqs):
+                                                                   generation_start, max_num_seqs, d_model):
     """anchor_ratio = 1.0: every affix token is recomputed, so refresh logits must equal the full-recompute
-    baseline.  max_num_seqs = 4 exercises query-side relocation, 1 the materialised / key-side path."""
-    cfg, model = _model(device, seed=7)
+    baseline.  max_num_seqs = 4 exercises query-side relocation, 1 the materialised / key-side path.  d_model 64
+    is the reference tests' own tiny configuration (4 heads of 16); 384 gives heads of 96."""
+    cfg, model = _model(device, seed=7, d_model=d_model)
 
     def serve(enable):
         return _serve(cfg, recompute_batch_size=1, gen_length=2, block_length=2, max_num_seqs=max_num_seqs,
@@ -234,11 +236,12 @@ def test_hip_graph_replay_of_refinement_steps_gives_the_same_tokens(device, use_
         assert all(63 not in g for g in replayed)
 
 
+@pytest.mark.parametrize("d_model", [256, 64])
 @pytest.mark.parametrize("placement", ["prefix", "infix"])
-def test_batched_probe_at_admission_selects_the_same_anchors(device, placement):
+def test_batched_probe_at_admission_selects_the_same_anchors(device, placement, d_model):
     """Config.anchor_selection_batch_size = 0 probes all admitted requests in one forward instead of one forward
     per request (the reference's choice, model_runner.py:873): same anchors, same generated tokens."""
-    cfg, model = _model(device, seed=3)
+    cfg, model = _model(device, seed=3, d_model=d_model)
     affix = list(range(20, 32))
 
     def make(i):

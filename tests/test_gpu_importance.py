@@ -31,7 +31,8 @@ def _case(device, H, Hkv, D, A, mask_counts, shifts, slot0=0, dtype=torch.bfloat
     return imp, want, (q, kc, rows, cu, args)
 
 
-@pytest.mark.parametrize("H,Hkv,D", [(4, 4, 128), (8, 2, 128), (28, 4, 128), (4, 2, 64)])
+@pytest.mark.parametrize("H,Hkv,D", [(4, 4, 128), (8, 2, 128), (28, 4, 128), (4, 2, 64), (4, 4, 16), (4, 2, 32),
+                                     (6, 2, 96), (4, 2, 160), (4, 4, 208), (2, 1, 256)])
 def test_importance_matches_oracle(device, H, Hkv, D):
     _case(device, H, Hkv, D, A=203, mask_counts=[32, 0, 17, 64, 1], shifts=[0, 3, 40, 7, 0], slot0=5, seed=H)
 

@@ -13,7 +13,7 @@ def _bits(t):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-@pytest.mark.parametrize("H,H_kv,D", [(32, 32, 128), (28, 4, 128), (4, 2, 64)])
+@pytest.mark.parametrize("H,H_kv,D", [(32, 32, 128), (28, 4, 128), (4, 2, 64), (4, 4, 16), (6, 2, 160), (3, 1, 96), (5, 5, 256)])
 def test_rope_qk_scatter_bit_exact(device, dtype, H, H_kv, D):
     g = torch.Generator().manual_seed(0)
     N, NB, BS = 53, 5, 16
