@@ -318,6 +318,38 @@ def test_anchor_recompute_config_against_oracle_on_a_head_subset(device):
     _close(got, want)
 
 
+def test_anchor_recompute_config_full_size_against_library_attention_on_device(device):
+    """All 32 heads of the anchor-recompute configuration (the benchmark's call): every request against
+    F.scaled_dot_product_attention in fp32 on the gathered K/V (a library routine, independent of the oracle), plus
+    the properties that need no reference: a duplicated batch gives the same bits, and permuting each request's
+    key order changes the result by rounding only."""
+    import torch.nn.functional as F
+    w = attention_batch(seed=0)
+    H = Hkv = 32
+    D, BS = 128, 256
+    g = torch.Generator(device=device).manual_seed(0)
+    S = w["num_blocks"] * BS
+    q = (torch.randn(int(w["cu_q"][-1]), H, D, generator=g, device=device) / D ** 0.5).to(torch.bfloat16)
+    kc = (torch.randn(S, Hkv, D, generator=g, device=device) / D ** 0.5).to(torch.bfloat16)
+    vc = (torch.randn(S, Hkv, D, generator=g, device=device) / D ** 0.5).to(torch.bfloat16)
+    cu_q, cu_k, slots = w["cu_q"].to(device), w["cu_k"].to(device), w["slot_map"].to(device)
+    kc4, vc4 = kc.view(-1, BS, Hkv, D), vc.view(-1, BS, Hkv, D)
+    got = ops.acache_attention(q, kc4, vc4, cu_q, cu_k, slots)
+    worst = 0.0
+    for b in range(len(w["q_lens"])):
+        q0, q1, k0, k1 = int(cu_q[b]), int(cu_q[b + 1]), int(cu_k[b]), int(cu_k[b + 1])
+        idx = slots[k0:k1].long()
+        want = F.scaled_dot_product_attention(q[q0:q1].float().transpose(0, 1), kc[idx].float().transpose(0, 1),
+                                              vc[idx].float().transpose(0, 1)).transpose(0, 1)
+        worst = max(worst, (got[q0:q1].float() - want).abs().max().item())
+    assert worst <= ATOL, worst
+    assert torch.equal(ops.acache_attention(q, kc4, vc4, cu_q, cu_k, slots), got)
+    perm = torch.cat([int(cu_k[b]) + torch.randperm(int(cu_k[b + 1] - cu_k[b]), device=device)
+                      for b in range(len(w["q_lens"]))])
+    got_p = ops.acache_attention(q, kc4, vc4, cu_q, cu_k, slots[perm])
+    assert (got_p.float() - got.float()).abs().max().item() <= 4e-3
+
+
 def test_block_table_variants(device):
     """baseline_ragged_attention / baseline_decode_attention geometry of tests/test_attention_kernels.py:371-476,
     checked against dense attention over the un-paged K/V."""
