@@ -152,6 +152,17 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
     qo_bytes = 2 * total_q * H * D * 2
     tflops = flops / (avg_ms * 1e-3) / 1e12
     extra = {"cpu_baseline": cpu_attention_baseline(torch, q, kc, vc, w)} if cpu_baseline else {}
+    # what the library GEMM reaches on a large square bf16 product on the same box: the practical matrix-core
+    # reference next to the nominal peak (reported, not used in `frac`)
+    n = 8192
+    ga = torch.randn(n, n, device=device).to(torch.bfloat16)
+    gb = torch.randn(n, n, device=device).to(torch.bfloat16)
+    for _ in range(3):
+        torch.matmul(ga, gb)
+    torch.cuda.synchronize()
+    gemm_ms = _event_times_ms(lambda: torch.matmul(ga, gb), 10, torch)
+    gemm_tflops = 2 * n ** 3 / (sum(gemm_ms) / len(gemm_ms) * 1e-3) / 1e12
+    del ga, gb
     return {
         **extra,
         "metric": "anchor-recompute attn TFLOP/s", "value": round(tflops, 1), "unit": "TFLOP/s",
@@ -163,7 +174,8 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
                      "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["attention"],
                      "kernel": "varlen_attn_dma_kernel<bf16,128,plain>", "algorithmic_flops": flops,
                      "algorithmic_bytes": kv_bytes + qo_bytes,
-                     "achieved_GBps": round((kv_bytes + qo_bytes) / (avg_ms * 1e-3) / 1e9, 1)},
+                     "achieved_GBps": round((kv_bytes + qo_bytes) / (avg_ms * 1e-3) / 1e9, 1),
+                     "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)},
     }
 
 
@@ -223,6 +235,14 @@ def kernel_sweep(torch, device, ops, steps):
     dst = torch.empty_like(src)
     row("device copy (torch copy_)", timed(lambda: dst.copy_(src)), 2 * (1 << 32), "4 GiB read + 4 GiB written")
     del src, dst
+    # the practical matrix-core reference: what the library GEMM reaches on a large square bf16 product
+    n = 8192
+    a = torch.randn(n, n, device=device).to(torch.bfloat16)
+    b = torch.randn(n, n, device=device).to(torch.bfloat16)
+    us = timed(lambda: torch.matmul(a, b))
+    out.append({"kernel": "library GEMM (torch.matmul, bf16)", "us": round(us, 1), "TFLOPs": round(2 * n ** 3 / us / 1e6, 1),
+                "flops": 2 * n ** 3, "workload": "8192 x 8192 x 8192"})
+    del a, b
 
     # configs[2]: Dream shape (28 layers, 4 KV heads, D 128), anchors of 16 requests
     w = anchor_batch(seed=0)
