@@ -171,7 +171,7 @@ __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], floa
                                                   float c, int n_valid, int lg) {
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
-    if (MASKED) {
+    if (MASKED && n_valid < 16 * NT) {  // wave-uniform: full tiles skip the masking code
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
