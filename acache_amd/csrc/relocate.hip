@@ -220,7 +220,7 @@ static int launch_relocate(const RelocateParams &p, hipStream_t stream) {
   const int64_t rows = p.T * p.H_kv;
   if (rows == 0 || p.L == 0) return 0;
   const int64_t gx = (rows + RPB - 1) / RPB;
-  if (gx > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "relocate: too many rows (%lld)", (long long)rows);
+  if (gx > 0x7fffffffLL || p.L > 65535) return fail(ACACHE_E_SHAPE, "relocate: too many rows (%lld) or layers", (long long)rows);
   // One layer per block measured best on MI355X (5.9 TB/s against 5.4 TB/s with two
   // layers per block): the extra blocks hide more latency than deeper per-lane
   // unrolling, and token-fastest block order keeps concurrent blocks on

@@ -98,6 +98,7 @@ __global__ __launch_bounds__(256) void slot_layout_kernel(SlotLayoutParams p) {
   const int k0 = p.cu_anchor[b];
   const int K = p.cu_anchor[b + 1] - k0;
   const int r0 = p.cu_rec[b];
+  const int rec_len = p.cu_rec[b + 1] - r0;  // K + len - (a_hi - a_lo) when the inputs are consistent
   const int32_t *anc = p.anchors + k0;
   for (int pos = blockIdx.x * 256 + threadIdx.x; pos < len; pos += gridDim.x * 256) {
     int priv = -1, rank = -1;
@@ -120,8 +121,10 @@ __global__ __launch_bounds__(256) void slot_layout_kernel(SlotLayoutParams p) {
       const int blk = priv / p.block_size;
       const int id = blk < p.max_blocks ? p.tables[(int64_t)b * p.max_blocks + blk] : -1;
       slot = id < 0 ? -1 : id * p.block_size + (priv - blk * p.block_size);
-      p.recompute_pos[r0 + rank] = pos;
-      p.recompute_slots[r0 + rank] = slot;
+      if (rank < rec_len) {  // never write past this request's share, whatever the anchor list holds
+        p.recompute_pos[r0 + rank] = pos;
+        p.recompute_slots[r0 + rank] = slot;
+      }
     }
     p.read_slots[t0 + pos] = slot;
   }
@@ -161,8 +164,8 @@ extern "C" int acache_kv_scatter(
   p.src_layer_bytes = src_layer_stride * es; p.cache_layer_bytes = cache_layer_stride * es;
   p.chunks_per_token = (int32_t)(tok * es / 16); p.L = L;
   const int64_t gx = (N * p.chunks_per_token + 255) / 256;
-  if (gx > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "kv_scatter: too many rows");
   constexpr int LPB = 2;
+  if (gx > 0x7fffffffLL || (L + LPB - 1) / LPB > 65535) return fail(ACACHE_E_SHAPE, "kv_scatter: too many rows or layers");
   dim3 grid((unsigned)gx, (unsigned)((L + LPB - 1) / LPB));
   hipLaunchKernelGGL(scatter_kernel<LPB>, grid, dim3(256), 0, (hipStream_t)stream, p);
   return launch_status("scatter_kernel");
