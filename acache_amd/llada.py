@@ -107,14 +107,47 @@ class LLaDABlock(nn.Module):
         self.ff_out = nn.Linear(config.mlp_hidden_size, d, bias=False)
         self.rotary_emb = RotaryEmbedding(config)
         self.attn = Attention(h, self.head_dim, hkv)
+        self._fused = {}
+
+    def _fuse(self, name, linears):
+        """One weight (and bias) for several projections of the same input: the parameters of ``linears`` become
+        views of one concatenated tensor, so the state dict keeps the reference's names and shapes while the
+        forward runs a single, wider GEMM.  Rebuilt when the parameters have been moved or replaced."""
+        first = linears[0].weight
+        cached = self._fused.get(name)
+        if cached is None or cached[0].data_ptr() != first.data_ptr() or cached[0].dtype != first.dtype:
+            with torch.no_grad():
+                w = torch.cat([lin.weight for lin in linears]).contiguous()
+                b = torch.cat([lin.bias for lin in linears]).contiguous() if linears[0].bias is not None else None
+                row = 0
+                for lin in linears:
+                    n = lin.weight.shape[0]
+                    lin.weight.data = w[row:row + n]
+                    if b is not None:
+                        lin.bias.data = b[row:row + n]
+                    row += n
+            cached = self._fused[name] = (w, b)
+        return cached
+
+    @staticmethod
+    def _hooked(*linears):
+        # a projection somebody observes (forward hooks) keeps its own forward call
+        return any(lin._forward_hooks or lin._forward_pre_hooks for lin in linears)
 
     def forward(self, x, position_ids, max_pos):
         h, hkv, hd = self.config.n_heads, self.config.effective_n_kv_heads, self.head_dim
         y = self.attn_norm(x)
         lead = y.shape[:-1]
-        q = self.q_proj(y).view(*lead, h, hd)
-        k = self.k_proj(y).view(*lead, hkv, hd)
-        v = self.v_proj(y).view(*lead, hkv, hd)
+        if y.is_cuda and not torch.is_grad_enabled() and not self._hooked(self.q_proj, self.k_proj, self.v_proj):
+            # q, k and v are column views of one projection (the kernels take token strides)
+            qkv = F.linear(y, *self._fuse("qkv", (self.q_proj, self.k_proj, self.v_proj)))
+            q = qkv[..., :h * hd].view(*lead, h, hd)
+            k = qkv[..., h * hd:(h + hkv) * hd].view(*lead, hkv, hd)
+            v = qkv[..., (h + hkv) * hd:].view(*lead, hkv, hd)
+        else:
+            q = self.q_proj(y).view(*lead, h, hd)
+            k = self.k_proj(y).view(*lead, hkv, hd)
+            v = self.v_proj(y).view(*lead, hkv, hd)
         if self.config.rope and q.is_cuda:
             # rotary application and the K/V cache write in one launch (q and k are rotated in place)
             sin, cos = self.rotary_emb.get_rotary_embedding(max_pos or self.config.max_sequence_length, q.device)
@@ -128,6 +161,10 @@ class LLaDABlock(nn.Module):
             o = self.attn(q, k, v)
         x = x + self.attn_out(o.reshape(*lead, h * hd))
         y = self.ff_norm(x)
+        if y.is_cuda and not torch.is_grad_enabled() and not self._hooked(self.ff_proj, self.up_proj):
+            m = self.config.mlp_hidden_size
+            gu = F.linear(y, *self._fuse("gate_up", (self.ff_proj, self.up_proj)))
+            return x + self.ff_out(F.silu(gu[..., :m]) * gu[..., m:])
         return x + self.ff_out(F.silu(self.ff_proj(y)) * self.up_proj(y))
 
 
