@@ -269,3 +269,50 @@ def test_batched_probe_at_admission_selects_the_same_anchors(device, placement, 
         assert calls == {1: [1] * 5, 0: [5], 3: [3, 2]}[probe_batch]
     assert results[0] == results[1] == results[2]
     assert all(len(a) == 5 for a in results[0][0])          # ceil(0.4 * 12) anchors per request
+
+
+def test_merged_projections_keep_the_state_dict_and_follow_parameter_updates(device):
+    """q / k / v (and gate / up) run as one GEMM whose weight the separate projections' parameters are views of:
+    same state-dict names and shapes, loading new weights afterwards takes effect, and a hooked projection falls
+    back to its own forward call."""
+    cfg, model = _model(device, seed=5)
+    ids = torch.randint(2, 60, (2, 12), device=device)
+    pos = torch.arange(12, device=device).expand(2, 12)
+    runner = ModelRunner(model, _serve(cfg, enable_acache=False))      # gives the attention modules a cache
+
+    def forward():
+        seqs = [Sequence(ids[i].tolist(), gen_length=4, cache_block_size=8, block_length=4, mask_id=63) for i in range(2)]
+        for s in seqs:
+            runner.block_manager.allocate(s)
+            s.finalize_slot_mapping()
+        with torch.inference_mode():
+            flat_ids, flat_pos, _, _ = runner.prepare_caching(seqs)
+            out = model(flat_ids, position_ids=flat_pos).logits.float()
+        reset_context()
+        for s in seqs:
+            runner.block_manager.deallocate(s)
+        return out
+
+    keys_before = {k: tuple(v.shape) for k, v in model.state_dict().items()}
+    merged = forward()
+    block = model.model.transformer["blocks"][0]
+    w_qkv = block._fused["qkv"][0]
+    assert block.q_proj.weight.data_ptr() == w_qkv.data_ptr()          # parameters alias the merged weight
+    assert {k: tuple(v.shape) for k, v in model.state_dict().items()} == keys_before
+    # a hooked projection is called on its own: same result up to GEMM rounding
+    seen = []
+    hook = block.k_proj.register_forward_hook(lambda m, i, o: seen.append(tuple(o.shape)))
+    separate = forward()
+    hook.remove()
+    assert seen and seen[0][-1] == cfg.d_model
+    torch.testing.assert_close(separate, merged, rtol=2e-2, atol=2e-2)
+    # new weights loaded through the usual interface are what the merged GEMM uses
+    state = {k: (torch.randn_like(v) * 0.08 if v.dim() > 1 else v.clone()) for k, v in model.state_dict().items()}
+    model.load_state_dict(state)
+    assert block.q_proj.weight.data_ptr() == w_qkv.data_ptr()
+    assert torch.equal(w_qkv[: cfg.d_model], state["model.transformer.blocks.0.q_proj.weight"])
+    changed = forward()
+    assert (changed - merged).abs().max().item() > 1e-2
+    hook = block.k_proj.register_forward_hook(lambda m, i, o: None)
+    torch.testing.assert_close(forward(), changed, rtol=2e-2, atol=2e-2)
+    hook.remove()
