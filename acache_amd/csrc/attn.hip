@@ -948,6 +948,14 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     const int r = idx - tile * heads_per_xcd;
     kvh = xcd * (p.H_kv >> 3) + r / group;
     hg = r % group;
+  } else if (8 % p.H_kv == 0) {
+    // fewer KV heads than XCDs (1, 2 or 4): 8 / H_kv XCDs share a KV head and deal its query tiles out
+    // round-robin in longest-first order, so each of them gets the same mix of long and short tiles
+    const int xcds_per_head = 8 / p.H_kv;
+    kvh = xcd / xcds_per_head;
+    tile = (idx / group) * xcds_per_head + xcd % xcds_per_head;
+    if (tile >= p.num_tiles) return;
+    hg = idx % group;
   } else {
     const int w = xcd * per_xcd + idx;
     if (w >= p.num_tiles * p.H) return;
@@ -982,6 +990,11 @@ static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStrea
   p.num_tiles = (int32_t)((total_q + BM - 1) / BM) + p.B;
   int64_t blocks = (int64_t)p.num_tiles * p.H;
   blocks = (blocks + 7) / 8 * 8;  // the XCD remap needs a multiple of 8
+  if (p.H_kv < 8 && 8 % p.H_kv == 0 && mode != MODE_KEY_SIDE) {
+    // 8 / H_kv XCDs per KV head, each walking every (8 / H_kv)-th query tile of all heads of the group
+    const int xcds_per_head = 8 / p.H_kv;
+    blocks = 8 * (((int64_t)p.num_tiles + xcds_per_head - 1) / xcds_per_head) * (p.H / p.H_kv);
+  }
   if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
   dim3 grid((unsigned)blocks), block(256);
   switch (mode) {
