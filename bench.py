@@ -180,15 +180,19 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
 
 
 def attention_shape_sweep(torch, device, ops, steps):
-    """Uniform-shape runs of the same attention kernel (MHA, 32 heads, D = 128, bf16, identity slot map): decode-like
-    shapes are bound by streaming K/V once, long-query shapes by the matrix core.  Median of per-call HIP event pairs."""
-    H, D = 32, 128
+    """Uniform-shape runs of the same attention kernel (D = 128, bf16, identity slot map): decode-like shapes are
+    bound by streaming K/V once, long-query shapes by the matrix core.  LLaDA heads (32, MHA) and Dream heads
+    (28 over 4 KV heads).  Median of per-call HIP event pairs."""
+    D = 128
     rows = []
-    for B, q, kv in ((16, 32, 1400), (16, 32, 2800), (64, 32, 1400), (16, 128, 1400), (16, 600, 1400), (4, 4096, 4096)):
+    shapes = [(16, 32, 1400, 32, 32), (16, 32, 2800, 32, 32), (64, 32, 1400, 32, 32), (16, 128, 1400, 32, 32),
+              (16, 600, 1400, 32, 32), (4, 4096, 4096, 32, 32), (16, 32, 1400, 28, 4), (16, 232, 1400, 28, 4),
+              (16, 600, 1400, 28, 4)]
+    for B, q, kv, H, Hkv in shapes:
         S = B * kv
         Q = (torch.randn(B * q, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
-        K = (torch.randn(S, 1, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
-        V = (torch.randn(S, 1, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        K = (torch.randn(S, 1, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        V = (torch.randn(S, 1, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
         cu_q = torch.arange(0, (B + 1) * q, q, dtype=torch.int32, device=device)
         cu_k = torch.arange(0, (B + 1) * kv, kv, dtype=torch.int32, device=device)
         slots = torch.arange(S, dtype=torch.int32, device=device)
@@ -202,9 +206,9 @@ def attention_shape_sweep(torch, device, ops, steps):
             b.record()
         torch.cuda.synchronize()
         ms = statistics.median(a.elapsed_time(b) for a, b in pairs)
-        kv_bytes = 2 * S * H * D * 2
-        rows.append({"B": B, "q": q, "kv": kv, "us": round(ms * 1e3, 1), "TFLOPs": round(4 * H * D * B * q * kv / ms / 1e9, 0),
-                     "kv_GBps": round(kv_bytes / ms / 1e6, 0)})
+        kv_bytes = 2 * S * Hkv * D * 2
+        rows.append({"B": B, "q": q, "kv": kv, "H": H, "H_kv": Hkv, "us": round(ms * 1e3, 1),
+                     "TFLOPs": round(4 * H * D * B * q * kv / ms / 1e9, 0), "kv_GBps": round(kv_bytes / ms / 1e6, 0)})
     print(json.dumps({"attention_shape_sweep": rows}))
 
 
