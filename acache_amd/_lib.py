@@ -47,6 +47,10 @@ SIGNATURES = {
     "acache_build_slot_layout": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         c_int32, c_int32, c_int32, c_int32, c_int64, c_void_p]),
+    "acache_swiglu": (c_int32, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int32, c_void_p]),
+    "acache_add_rms_norm": (c_int32, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_float,
+        c_int32, c_void_p]),
     "acache_varlen_attn": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
         c_float,

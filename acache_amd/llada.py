@@ -134,9 +134,22 @@ class LLaDABlock(nn.Module):
         # a projection somebody observes (forward hooks) keeps its own forward call
         return any(lin._forward_hooks or lin._forward_pre_hooks for lin in linears)
 
-    def forward(self, x, position_ids, max_pos):
+    def fusable(self, x) -> bool:
+        """The merged-launch form of the block applies: GPU inference with nobody observing the sub-modules."""
+        return (x.is_cuda and not torch.is_grad_enabled() and self.config.rope and not self._forward_hooks
+                and not self._forward_pre_hooks
+                and not self._hooked(self.attn_norm, self.ff_norm, self.q_proj, self.k_proj, self.v_proj,
+                                     self.attn_out, self.ff_proj, self.up_proj, self.ff_out))
+
+    def forward(self, x, position_ids, max_pos, pending=None, defer_residual=False):
+        """``pending``: a residual term the previous block left un-added; it is folded into this block's first
+        layer norm.  ``defer_residual``: return ``(x, mlp_out)`` instead of their sum, for the next block (or the
+        final norm) to fold in the same way.  Both only with ``fusable(x)``; the plain call is the reference's."""
         h, hkv, hd = self.config.n_heads, self.config.effective_n_kv_heads, self.head_dim
-        y = self.attn_norm(x)
+        if pending is not None or defer_residual:
+            x, y = ops.add_rms_norm(x, pending, self.attn_norm.weight, self.attn_norm.eps)
+        else:
+            y = self.attn_norm(x)
         lead = y.shape[:-1]
         if y.is_cuda and not torch.is_grad_enabled() and not self._hooked(self.q_proj, self.k_proj, self.v_proj):
             # q, k and v are column views of one projection (the kernels take token strides)
@@ -159,12 +172,17 @@ class LLaDABlock(nn.Module):
             if self.config.rope:
                 q, k = self.rotary_emb(q, k, position_ids, max_pos)
             o = self.attn(q, k, v)
-        x = x + self.attn_out(o.reshape(*lead, h * hd))
-        y = self.ff_norm(x)
-        if y.is_cuda and not torch.is_grad_enabled() and not self._hooked(self.ff_proj, self.up_proj):
-            m = self.config.mlp_hidden_size
+        attn = self.attn_out(o.reshape(*lead, h * hd))
+        fused = x.is_cuda and not torch.is_grad_enabled() and not self._hooked(self.ff_norm, self.ff_proj, self.up_proj)
+        if fused:
+            # residual add and layer norm in one pass over the row, then gate and up as one GEMM and SwiGLU in
+            # one pass
+            x, y = ops.add_rms_norm(x, attn, self.ff_norm.weight, self.ff_norm.eps)
             gu = F.linear(y, *self._fuse("gate_up", (self.ff_proj, self.up_proj)))
-            return x + self.ff_out(F.silu(gu[..., :m]) * gu[..., m:])
+            mlp = self.ff_out(ops.swiglu(gu, self.config.mlp_hidden_size))
+            return (x, mlp) if defer_residual else x + mlp
+        x = x + attn
+        y = self.ff_norm(x)
         return x + self.ff_out(F.silu(self.ff_proj(y)) * self.up_proj(y))
 
 
@@ -184,11 +202,22 @@ class LLaDAModel(nn.Module):
             position_ids = torch.arange(input_ids.shape[-1], device=input_ids.device).expand_as(input_ids)
         max_pos = self.config.max_sequence_length
         x = self.transformer["wte"](input_ids)
-        for block in self.transformer["blocks"]:
-            x = block(x, position_ids, max_pos)
-        if not compute_logits:
-            return SimpleNamespace(logits=None, hidden_states=x)
-        x = self.transformer["ln_f"](x)
+        blocks = self.transformer["blocks"]
+        ln_f = self.transformer["ln_f"]
+        if len(blocks) and all(block.fusable(x) for block in blocks) and not ln_f._forward_hooks:
+            # every residual add rides along with the layer norm that follows it
+            pending = None
+            for block in blocks:
+                x, pending = block(x, position_ids, max_pos, pending=pending, defer_residual=True)
+            if not compute_logits:
+                return SimpleNamespace(logits=None, hidden_states=x + pending)
+            _, x = ops.add_rms_norm(x, pending, ln_f.weight, ln_f.eps)
+        else:
+            for block in blocks:
+                x = block(x, position_ids, max_pos)
+            if not compute_logits:
+                return SimpleNamespace(logits=None, hidden_states=x)
+            x = ln_f(x)
         if logits_keep_indices is not None:  # logits of the listed ragged rows only
             x = x.reshape(-1, x.shape[-1]).index_select(0, logits_keep_indices)
         return SimpleNamespace(logits=self.transformer["ff_out"](x))

@@ -267,6 +267,45 @@ def argmax_confidence(logits: torch.Tensor, picks: torch.Tensor | None = None):
     return token.view(logits.shape[:-1]), conf.view(logits.shape[:-1])
 
 
+def swiglu(gate_up: torch.Tensor, hidden: int) -> torch.Tensor:
+    """``silu(gate_up[..., :hidden]) * gate_up[..., hidden:]`` of a merged gate / up projection in one pass (the
+    MLP activation of the decoder block: ``act(ff_proj(x)) * up_proj(x)``)."""
+    assert gate_up.is_cuda and gate_up.shape[-1] == 2 * hidden and gate_up.stride(-1) == 1
+    flat = gate_up.reshape(-1, 2 * hidden)
+    out = torch.empty(flat.shape[0], hidden, dtype=gate_up.dtype, device=gate_up.device)
+    lib = _lib.load()
+    with torch.cuda.device(gate_up.device):
+        rc = lib.acache_swiglu(_ptr(out), _ptr(flat), flat.shape[0], hidden,
+                               flat.stride(0) if flat.shape[0] > 1 else 2 * hidden, hidden, _code(flat), _stream(flat))
+    _lib.check(rc, "swiglu")
+    return out.view(*gate_up.shape[:-1], hidden)
+
+
+def add_rms_norm(x: torch.Tensor, delta: torch.Tensor | None, weight: torch.Tensor, eps: float):
+    """Residual add and RMS layer norm in one pass: returns ``(x + delta, norm(x + delta))`` where
+    ``norm(s) = s * rsqrt(mean(s^2) + eps) * weight`` (statistics in fp32, one rounding).  With ``delta`` None the
+    first element is ``x`` itself.  ``x``: ``[..., d]`` with contiguous rows; nothing is modified in place."""
+    d = x.shape[-1]
+    assert x.is_cuda and x.stride(-1) == 1 and weight.shape == (d,)
+    flat = x.reshape(-1, d)
+    M = flat.shape[0]
+    y = torch.empty(M, d, dtype=x.dtype, device=x.device)
+    w = (weight if weight.dtype == x.dtype else weight.to(x.dtype)).contiguous()
+    total = dl = None
+    if delta is not None:
+        assert delta.shape == x.shape and delta.dtype == x.dtype and delta.stride(-1) == 1
+        dl = delta.reshape(-1, d)
+        total = torch.empty(M, d, dtype=x.dtype, device=x.device)
+    stride = lambda t: t.stride(0) if M > 1 else d
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        rc = lib.acache_add_rms_norm(_ptr(total), _ptr(flat), _ptr(dl), _ptr(w), _ptr(y), M, d,
+                                     d, stride(flat), stride(dl) if dl is not None else d, d, float(eps),
+                                     _code(flat), _stream(flat))
+    _lib.check(rc, "add_rms_norm")
+    return (total.view(x.shape) if total is not None else x), y.view(x.shape)
+
+
 def affix_importance(
     importance: torch.Tensor,
     q: torch.Tensor,

@@ -328,6 +328,32 @@ int acache_varlen_attn(
     int64_t kv_slot_stride, int64_t kv_head_stride,
     void *stream);
 
+/*
+ * Two elementwise steps of the decoder block on either side of the attention path, for
+ * hosts that run the model through this library (the package's own LLaDA / Dream mirror
+ * does).  They sit outside the affix-reuse path proper; their reference counterparts are
+ * model code: the SwiGLU of the MLP, act(ff_proj(x)) * up_proj(x), and the residual add in
+ * front of the RMS layer norm (nano-vdllm/model/modeling_llada.py, block forward).
+ *
+ * acache_swiglu: out[t, j] = silu(gate_up[t, j]) * gate_up[t, m + j] for t < M, j < m, where a
+ * row of gate_up holds the gate projection followed by the up projection (one merged GEMM).
+ * silu in fp32, rounded to `dtype`, multiplied by the up value in fp32, rounded again (the
+ * roundings of the separate activation and multiply kernels).  m * sizeof(dtype) must be a
+ * multiple of 16; row strides in elements.
+ *
+ * acache_add_rms_norm: sum[t, :] = x[t, :] + delta[t, :] rounded to `dtype` (sum may be x itself;
+ * with delta == NULL the sum is x and nothing is written to `sum`, which may then be NULL),
+ * y[t, :] = sum[t, :] * rsqrt(mean(sum[t, :]^2) + eps) * weight[:], statistics in fp32, one
+ * rounding of y.  y may not overlap the other rows.  d * sizeof(dtype) a multiple of 16 and at
+ * most 16 KiB.
+ */
+int acache_swiglu(void *out, const void *gate_up, int64_t M, int64_t m,
+                  int64_t in_row_stride, int64_t out_row_stride, int32_t dtype, void *stream);
+int acache_add_rms_norm(void *sum, const void *x, const void *delta, const void *weight, void *y,
+                        int64_t M, int64_t d, int64_t sum_row_stride, int64_t x_row_stride,
+                        int64_t delta_row_stride, int64_t y_row_stride, float eps, int32_t dtype,
+                        void *stream);
+
 #ifdef __cplusplus
 }
 #endif
