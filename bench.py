@@ -267,6 +267,30 @@ def kernel_sweep(torch, device, ops, steps):
     starts = torch.tensor(w["affix_start"], dtype=torch.int32, device=device)
     row("topk_kernel (batch of 16, one launch)", timed(lambda: ops.topk_anchors(scores, cu_a, cu_k, n_anchor, offsets=starts)),
         4 * sum(w["A"]) + 8 * n_anchor, f"configs[2]: {sum(w['A'])} fp32 scores, {n_anchor} indices out")
+    # the same two steps in the reference's torch formulation on the host cores (one layer of the scatter)
+    import time as _time
+    cpu_scores = [t.clone() for t in w["scores"]]
+    def cpu_topk():
+        return [torch.topk(sc, k).indices.sort().values + a0 for sc, k, a0 in zip(cpu_scores, w["K"], w["affix_start"])]
+    ck, cv = key[0].cpu(), val[0].cpu()
+    ckc = torch.zeros(nblk * BS, Hkv, D, dtype=torch.bfloat16)
+    cvc = torch.zeros_like(ckc)
+    cslots = slots.cpu().long()
+    def cpu_scatter():
+        ckc.index_copy_(0, cslots, ck)
+        cvc.index_copy_(0, cslots, cv)
+    def cpu_timed(fn, n=7):
+        fn(); fn()
+        ts = []
+        for _ in range(n):
+            t0 = _time.perf_counter(); fn(); ts.append(_time.perf_counter() - t0)
+        return statistics.median(ts) * 1e6
+    us_topk, us_scatter = cpu_timed(cpu_topk), cpu_timed(cpu_scatter)
+    out.append({"kernel": "cpu baseline: torch.topk + sort per request", "us": round(us_topk, 1), "cores": torch.get_num_threads(),
+                "workload": "configs[2], same scores"})
+    out.append({"kernel": "cpu baseline: index_copy_ of K and V, one layer", "us": round(us_scatter, 1),
+                "GBps": round(2 * 2 * n_anchor * Hkv * D * 2 / us_scatter / 1e3, 2), "cores": torch.get_num_threads(),
+                "workload": f"configs[2], one of 28 layers ({n_anchor} rows)"})
     del key, val, kc, vc
 
     # the steps on either side of attention, LLaDA-8B shape
