@@ -110,7 +110,7 @@ class ModelRunner:
             return
         bs = int(self.config.cache_block_size)
         used = len(self.block_manager.used_block_ids)
-        cap = len(self.block_manager.blocks)
+        cap = self.block_manager.num_blocks
         timing["kv_cache_block_size"] = bs
         timing["kv_cache_block_bytes"] = int(self.kv_cache_block_bytes)
         timing["kv_cache_slot_bytes"] = int(self.kv_cache_block_bytes // bs)
@@ -241,10 +241,10 @@ class ModelRunner:
             self._relocated_affix_slot_offset = None
             return False
         need = self.shared_prefix_blocks
-        if len(bm.free_block_ids) < need + seq.num_cache_blocks:
+        if bm.num_free_blocks < need + seq.num_cache_blocks:
             return False
         end = self.shared_prefix_blocks + need
-        if any(not bm.blocks[i].is_free for i in range(self.shared_prefix_blocks, end)):
+        if end > bm.num_blocks or not all(bm.is_free(i) for i in range(self.shared_prefix_blocks, end)):
             return False
         bm.reserve_prefix(end)
         self._relocated_affix_slot_offset = self.shared_prefix_blocks * self.config.cache_block_size
@@ -516,7 +516,7 @@ class ModelRunner:
 
     def _collect_admissible_sequences(self, prompts, next_prompt_idx, current_batch_size, max_num_seqs):
         admissible = []
-        remaining = len(self.block_manager.free_block_ids)
+        remaining = self.block_manager.num_free_blocks
         while next_prompt_idx < len(prompts) and current_batch_size + len(admissible) < max_num_seqs:
             seq = prompts[next_prompt_idx]
             if seq.num_cache_blocks > remaining:

@@ -91,8 +91,13 @@ def test_block_manager_fifo_order_and_exhaustion():
     assert bm.can_allocate(c)
     bm.allocate(c)
     assert c.block_table == [3, 2]
+    assert not bm.is_free(3) and bm.num_free_blocks == 0
     with pytest.raises(AssertionError):
-        bm._allocate_block(3)
+        bm.allocate(c)                                  # a sequence that already owns blocks
+    d = Sequence(list(range(6)), gen_length=2, cache_block_size=4)
+    with pytest.raises(IndexError):
+        bm.allocate(d)                                  # empty pool, as the reference's free_block_ids[0]
+    assert d.block_table == []
 
 
 def test_anchor_budget_and_private_slot_accounting():
