@@ -38,6 +38,11 @@ SIGNATURES = {
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float,
         c_int32, c_int64, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
         c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
+    "acache_affix_importance_noalloc_max_bytes": (c_int64, []),
+    "acache_affix_importance_noalloc": (c_int32, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float,
+        c_int32, c_int64, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
+        c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "acache_topk_anchors": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),
     "acache_argmax_confidence": (c_int32, [

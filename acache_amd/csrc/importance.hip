@@ -17,6 +17,8 @@
 // Scores come from the matrix core (S^T = K Q^T, keys as rows, one query column per lane).  K and Q
 // fragments are loaded straight from global memory in operand layout (16 bytes per lane); nothing goes
 // through LDS and there is no barrier.
+#include <mutex>
+
 #include "common.h"
 #include "mma.h"
 
@@ -278,7 +280,8 @@ extern "C" int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_ro
   return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len);
 }
 
-extern "C" int acache_affix_importance(
+// Argument checks and the launches; `workspace` is caller memory or this library's file-scope scratch.
+static int importance_launch(
     float *importance, const void *q, const void *k_cache, const int32_t *mask_rows, const int32_t *cu_mask,
     const int32_t *affix_shifts, const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
     int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows, int32_t H,
@@ -354,4 +357,75 @@ extern "C" int acache_affix_importance(
 #undef ACACHE_SLABS
 #undef ACACHE_CASE
   return fail(ACACHE_E_SHAPE, "affix_importance: unsupported dtype / head_dim");
+}
+
+extern "C" int acache_affix_importance(
+    float *importance, const void *q, const void *k_cache, const int32_t *mask_rows, const int32_t *cu_mask,
+    const int32_t *affix_shifts, const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows, int32_t H,
+    int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t importance_stride, int64_t q_token_stride,
+    int64_t q_head_stride, int64_t kv_slot_stride, int64_t kv_head_stride, void *workspace, int64_t workspace_bytes,
+    void *stream) {
+  return importance_launch(importance, q, k_cache, mask_rows, cu_mask, affix_shifts, rope_cos, rope_sin, rope_rows, scale,
+                           affix_len, affix_slot0, B, total_mask_rows, max_mask_rows, H, H_kv, D, dtype, num_slots,
+                           importance_stride, q_token_stride, q_head_stride, kv_slot_stride, kv_head_stride, workspace,
+                           workspace_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The same call for callers that cannot allocate device memory (code under HIP graph capture, serving
+// loops, harnesses that forbid hipMalloc): the row statistics, per-head partial sums and re-rotated keys
+// live in a file-scope device array instead of a caller workspace.  Every GPU the library runs on holds
+// its own copy of the array at its own address until the process ends; the address is looked up once per
+// device and only that pointer is ever handed to kernels.  Nothing in the array has to start at zero:
+// every word a launch reads was written by an earlier launch of the same call.
+static __device__ __align__(256) unsigned char scratch[ACACHE_IMPORTANCE_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int scratch_of_current_device(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail((int)e, "affix_importance_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices)
+    return fail(ACACHE_E_RANGE, "affix_importance_noalloc: device %d outside the %d devices supported", dev, kMaxDevices);
+  std::lock_guard<std::mutex> guard(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(e != hipSuccess ? (int)e : ACACHE_E_NULL, "affix_importance_noalloc: hipGetSymbolAddress: %s",
+                  hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace
+
+extern "C" int64_t acache_affix_importance_noalloc_max_bytes(void) { return ACACHE_IMPORTANCE_SCRATCH_BYTES; }
+
+extern "C" int acache_affix_importance_noalloc(
+    float *importance, const void *q, const void *k_cache, const int32_t *mask_rows, const int32_t *cu_mask,
+    const int32_t *affix_shifts, const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows, int32_t H,
+    int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t importance_stride, int64_t q_token_stride,
+    int64_t q_head_stride, int64_t kv_slot_stride, int64_t kv_head_stride, void *stream) {
+  const int64_t need =
+      acache_affix_importance_workspace_bytes(total_mask_rows, B, H, H_kv, D, affix_len, affix_shifts != nullptr);
+  if (need > (int64_t)ACACHE_IMPORTANCE_SCRATCH_BYTES)
+    return fail(ACACHE_E_SHAPE,
+                "affix_importance_noalloc: this call needs %lld bytes of scratch, the built-in buffer holds %lld; "
+                "use acache_affix_importance with a caller workspace",
+                (long long)need, (long long)ACACHE_IMPORTANCE_SCRATCH_BYTES);
+  void *ws = nullptr;
+  const int rc = scratch_of_current_device(&ws);
+  if (rc) return rc;
+  return importance_launch(importance, q, k_cache, mask_rows, cu_mask, affix_shifts, rope_cos, rope_sin, rope_rows, scale,
+                           affix_len, affix_slot0, B, total_mask_rows, max_mask_rows, H, H_kv, D, dtype, num_slots,
+                           importance_stride, q_token_stride, q_head_stride, kv_slot_stride, kv_head_stride, ws,
+                           ACACHE_IMPORTANCE_SCRATCH_BYTES, stream);
 }

@@ -326,7 +326,10 @@ def affix_importance(
     For each request the [MASK] queries ``q[mask_rows[cu_mask[b]:cu_mask[b+1]]]`` attend to the cached affix keys
     ``k_cache`` slots ``affix_slot0 .. + affix_len`` (re-rotated by ``affix_shifts[b]``); the softmax runs over the
     affix keys only and its columns are summed over queries and heads (nano-vdllm/model_runner.py:730-773).
-    ``workspace``: optional uint8 scratch of ``affix_importance_workspace_bytes`` bytes, allocated here if absent.
+    ``workspace``: optional uint8 scratch of ``affix_importance_workspace_bytes`` bytes, allocated here if absent;
+    the string ``"builtin"`` selects ``acache_affix_importance_noalloc``, which keeps its scratch in a fixed device
+    array inside the library (allocates nothing; rejects calls that need more than that array holds; calls on
+    one GPU must not overlap).
     """
     Tq, H, D = q.shape
     H_kv = k_cache.shape[-2]
@@ -344,18 +347,26 @@ def affix_importance(
     shifts = _i32(affix_shifts, "affix_shifts") if relocate else None
     scale = softmax_scale if softmax_scale is not None else D ** -0.5
     lib = _lib.load()
+    common = (
+        _ptr(importance), _ptr(q), _ptr(kc), _ptr(rows), _ptr(cu), _ptr(shifts),
+        _ptr(rope_cos) if relocate else None, _ptr(rope_sin) if relocate else None,
+        rope_cos.shape[0] if relocate else 0, float(scale),
+        affix_len, affix_slot0, B, total, max_mask_rows, H, H_kv, D, _code(q), kc.shape[0],
+        importance.stride(0), q.stride(0), q.stride(1), kc.stride(0), kc.stride(1))
+    if isinstance(workspace, str):
+        if workspace != "builtin":
+            raise ValueError("workspace: a uint8 tensor, None or 'builtin'")
+        with torch.cuda.device(q.device):
+            rc = lib.acache_affix_importance_noalloc(*common, _stream(q))
+        _lib.check(rc, "affix_importance_noalloc")
+        return importance
     need = lib.acache_affix_importance_workspace_bytes(total, B, H, H_kv, D, affix_len, int(relocate))
     if workspace is None:
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     assert workspace.is_cuda and workspace.numel() * workspace.element_size() >= need
     with torch.cuda.device(q.device):
-        rc = lib.acache_affix_importance(
-            _ptr(importance), _ptr(q), _ptr(kc), _ptr(rows), _ptr(cu), _ptr(shifts),
-            _ptr(rope_cos) if relocate else None, _ptr(rope_sin) if relocate else None,
-            rope_cos.shape[0] if relocate else 0, float(scale),
-            affix_len, affix_slot0, B, total, max_mask_rows, H, H_kv, D, _code(q), kc.shape[0],
-            importance.stride(0), q.stride(0), q.stride(1), kc.stride(0), kc.stride(1),
-            _ptr(workspace), workspace.numel() * workspace.element_size(), _stream(q))
+        rc = lib.acache_affix_importance(*common, _ptr(workspace), workspace.numel() * workspace.element_size(),
+                                         _stream(q))
     _lib.check(rc, "affix_importance")
     return importance
 

@@ -8,15 +8,17 @@
  *
  * Conventions shared by every entry point
  *   - all data pointers are DEVICE pointers owned by the caller; nothing is
- *     allocated, freed or retained by the library (the one entry point that needs
- *     scratch memory, acache_affix_importance, takes it as a workspace argument);
+ *     allocated, freed or retained by the library (entry points that need scratch
+ *     memory take it as a workspace argument; acache_affix_importance_noalloc is the
+ *     one exception and says so);
  *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = the
  *     default stream) and the call returns without synchronising;
  *   - return value: 0 = enqueued; < 0 = argument error (ACACHE_E_*), nothing was
  *     launched; > 0 = the hipError_t reported by the launch;
  *   - acache_last_error() returns a thread-local, human readable description of
  *     the most recent non-zero return on the calling thread;
- *   - calls are re-entrant across distinct streams; no global mutable state;
+ *   - calls are re-entrant across distinct streams; no global mutable state
+ *     (except the built-in scratch of acache_affix_importance_noalloc);
  *   - strides and offsets are counted in ELEMENTS of `dtype`, never bytes;
  *   - slot = block_id * cache_block_size + offset_in_block: an index into the
  *     cache viewed as [num_slots, H_kv, D] (per layer).
@@ -199,6 +201,33 @@ int acache_affix_importance(
     int64_t importance_stride, int64_t q_token_stride, int64_t q_head_stride,
     int64_t kv_slot_stride, int64_t kv_head_stride,
     void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * acache_affix_importance for callers that cannot allocate device memory.
+ *
+ * No counterpart in the reference.  It exists for callers that may not call hipMalloc (or
+ * torch's allocator) around the probe: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid allocation.  Same arguments, arithmetic and results as
+ * acache_affix_importance, bit for bit, minus the workspace: the scratch is a file-scope device
+ * array of ACACHE_IMPORTANCE_SCRATCH_BYTES inside the library (one copy per GPU the library
+ * runs on, held until the process ends; its address is looked up on the first call on each
+ * device).  The call allocates and frees nothing.
+ *
+ * A call whose acache_affix_importance_workspace_bytes(...) exceeds the array is rejected with
+ * ACACHE_E_SHAPE before anything is launched.  All calls on one GPU share that GPU's array:
+ * calls that overlap in time on the same GPU (different streams or threads) race; serialise
+ * them.  The current device must be the one `stream` belongs to.
+ */
+#define ACACHE_IMPORTANCE_SCRATCH_BYTES (32 << 20)
+int64_t acache_affix_importance_noalloc_max_bytes(void);
+int acache_affix_importance_noalloc(
+    float *importance, const void *q, const void *k_cache,
+    const int32_t *mask_rows, const int32_t *cu_mask, const int32_t *affix_shifts,
+    const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows,
+    int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int64_t importance_stride, int64_t q_token_stride, int64_t q_head_stride,
+    int64_t kv_slot_stride, int64_t kv_head_stride, void *stream);
 
 /*
  * Per-request top-k anchor selection over ragged fp32 influence scores.
