@@ -24,6 +24,7 @@
 // Both share the softmax steps below, so they round identically.  HBM traffic per
 // call: K and V rows once per (request, kv head) when query tiles of one head share
 // an L2 (block indices are mapped so that they land on the same XCD), Q once, O once.
+#include <stdlib.h>
 #include "attn_common.h"
 
 namespace acache {
@@ -318,10 +319,10 @@ __global__ __launch_bounds__(256, RAGGED ? 1 : 2) void varlen_attn_kernel(AttnPa
 
     // online softmax; P^T packed straight into the B operand of the PV product
     vec16 pf[NQ16][NS];
-    softmax_reference<NQ16, NT, DT, true>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
+    softmax_reference<NQ16, NQ16, NT, DT, true>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
     static_assert(NS == 2, "two 32-key slabs per tile");
-    softmax_probs_slab<M, 0>(s_acc, m_run, l_acc, pf, ones, c);
-    softmax_probs_slab<M, 1>(s_acc, m_run, l_acc, pf, ones, c);
+    softmax_probs_slab<M, 0, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
+    softmax_probs_slab<M, 1, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
 
     // O^T += V^T P^T ; lane reads V^T[16*dt + li][keys of slab s, group lg]
 #pragma unroll
@@ -383,12 +384,26 @@ __global__ __launch_bounds__(256, RAGGED ? 1 : 2) void varlen_attn_kernel(AttnPa
 // 4*j + i/4, j = 0..3.  With lane l pointing at V[row0 + l/4][d0 + 4*(l%4)] lane i
 // gets V[row0 + 0..3][d0 + i]: four keys of one column, i.e. half of an MFMA
 // A-operand of V^T.
-// One query tile of one (request, head): the four waves take WQ = 16 * NQ16 query rows each, starting at
-// row q_tile0 of the request, and stream the request's K/V through the LDS ring.
-template <int DTYPE, int D, int NQ16, int MODE>
-__device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0, char *lds_v0, char *lds_k1,
-                                              char *lds_v1, int b, int q_begin, int q_len, int q_tile0, int head,
-                                              int kvh) {
+// Partial results of a (query tile, head) unit whose key tiles were dealt to several workgroups: every
+// part leaves its un-normalised O^T accumulators, running reference m and running sum l in its workspace
+// slot, in register order (thread-major, 16 bytes per thread and register quad, so the stores coalesce).
+constexpr int kSkThreads = 256;
+constexpr int kSkAccBytes = kSkThreads * 16 * 16;            // 2 query tiles x 8 d tiles x 16 B per thread
+constexpr int kSkSlotBytes = kSkAccBytes + kSkThreads * 4 * 4;  // + (m, l) of the two query tiles
+constexpr int kSkCounterAlign = 4096;
+
+// Key tiles [t_begin, t_end) of one query tile of one (request, head): the four waves take WQ = 16 * NQ16 query
+// rows each, starting at row q_tile0 of the request, and stream the tiles through the LDS ring.
+// nparts == 1: the range is the whole unit and the result goes to `out`.  nparts > 1: the unit's tiles were dealt
+// to nparts consecutive workgroups (this one holds part `part`, the first one has global index first_gid); every
+// part writes its partial state to its workspace slot and bumps the unit's counter, and the part that finds
+// all the others already there merges them in part order (so the result does not depend on arrival order),
+// resets the counter and writes `out`.  Nobody waits for anybody.
+template <int DTYPE, int D, int NQ16, int MODE, int NW = 4>
+__device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0, char *lds_v0, char *lds_k1,
+                                              char *lds_v1, int *lds_flag, int b, int q_begin, int q_len,
+                                              int q_tile0, int head, int kvh, int t_begin, int t_end, int nparts,
+                                              int part, int first_gid) {
   constexpr int BN = 64;
   constexpr int WQ = 16 * NQ16;
   constexpr int KS = D / 32;
@@ -399,12 +414,17 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
   constexpr int CH = ROW_BYTES / 16;          // chunks per row: 16 (D=128) or 8 (D=64)
   constexpr int RW = 256 / ROW_BYTES;         // rows per bank window: 1 or 2
   constexpr int RPI = 64 / CH;                // rows per DMA instruction: 4 or 8
-  constexpr int WAVE_ROWS = BN / 4;           // 16 rows of every tile belong to each wave
+  constexpr int WAVE_ROWS = BN / NW;          // rows of every tile that each of the NW waves copies (16 or 8)
+  constexpr int THREADS = 64 * NW;
   constexpr int NI = WAVE_ROWS / RPI;         // DMA instructions per wave, tile and tensor: 4 or 2
   constexpr int TILE_BYTES = BN * ROW_BYTES;
   using M = Mma<DTYPE>;
   typedef short s16x4 __attribute__((ext_vector_type(4)));
-  const int tid = threadIdx.x;
+  // An opaque zero ties the lane-derived address constants below to this call: otherwise the compiler hoists them
+  // out of the persistent loop around it and spills them to keep them alive across units.
+  int opaque_zero;
+  asm volatile("s_mov_b32 %0, 0" : "=s"(opaque_zero));
+  const int tid = threadIdx.x + opaque_zero;
   const int lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, lg = lane >> 4;
   const int kv_begin = p.cu_k[b];
@@ -414,8 +434,11 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
   nq_valid = nq_valid < 0 ? 0 : (nq_valid > NQ16 ? NQ16 : nq_valid);
   char *out_base = p.out + (int64_t)q_begin * p.o_token_bytes + (int64_t)head * p.o_head_bytes;
 
+  // the previous unit of this workgroup may still be reading the ring (its output staging) and the flag word
+  __syncthreads();
+
   if (kv_len <= 0) {
-    for (int r = tid / CH; r < 4 * WQ; r += 256 / CH) {
+    for (int r = tid / CH; r < NW * WQ; r += THREADS / CH) {
       const int qr = q_tile0 + r;
       if (qr < q_len) store16(out_base + (int64_t)qr * p.o_token_bytes + (tid % CH) * 16, vec16{{0, 0, 0, 0}});
     }
@@ -431,8 +454,6 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
   }
 
   const int tiles_a = (shared_len + BN - 1) / BN;
-  const int tiles_b = (kv_len - shared_len + BN - 1) / BN;
-  const int n_tiles = tiles_a + tiles_b;
 
   // Query fragments (B operand).  Query-side mode scores the shared keys, which come first,
   // against the rotated query q' and everything after them against q itself; only one of the
@@ -457,7 +478,7 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
       }
     }
   };
-  load_q(MODE == MODE_QUERY_SIDE && tiles_a > 0);
+  load_q(MODE == MODE_QUERY_SIDE && t_begin < tiles_a);
 
   // ---- DMA bookkeeping: this lane's row and chunk inside each of its NI instructions
   const int dma_row0 = wave * WAVE_ROWS + lane / CH;   // + i*RPI
@@ -471,13 +492,13 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
   // ever placed in front of the MFMA work.
   int slot_a[NI], slot_b[NI];
   auto load_slots = [&](int t, int (&dst)[NI]) __attribute__((always_inline)) {
-    const TileRange tr = tile_range_of(t < n_tiles ? t : n_tiles - 1, tiles_a, shared_len, kv_len, BN);
+    const TileRange tr = tile_range_of(t < t_end ? t : t_end - 1, tiles_a, shared_len, kv_len, BN);
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       const int n = tr.n0 + dma_row0 + i * RPI;
       // rows past the end of the range read index 0 (kv_len > 0, always readable);
       // issue() ignores the value
-      dst[i] = p.slot_map[kv_begin + ((t < n_tiles && n < tr.n_end) ? n : 0)];
+      dst[i] = p.slot_map[kv_begin + ((t < t_end && n < tr.n_end) ? n : 0)];
     }
   };
   // Per-lane source addresses of row i of a tile, minus the slot term: base + swizzled chunk offset.
@@ -600,7 +621,7 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
     __builtin_amdgcn_s_setprio(0);
 
     copy_point(1);
-    softmax_reference<NQ16, NT, DT, MASKED>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
+    softmax_reference<NQ16, NQ16, NT, DT, MASKED>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
     copy_point(2);
 
     // O^T += V^T P^T, one 32-key slab at a time, so that the exponentials of the second slab
@@ -622,11 +643,11 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
           o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
       }
     };
-    softmax_probs_slab<M, 0>(s_acc, m_run, l_acc, pf, ones, c);
+    softmax_probs_slab<M, 0, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
     copy_point(3);
     __builtin_amdgcn_s_setprio(1);
     pv_slab(0);
-    softmax_probs_slab<M, 1>(s_acc, m_run, l_acc, pf, ones, c);
+    softmax_probs_slab<M, 1, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
     pv_slab(1);
     // Issue order: V fragments two d-tiles ahead of their use.
     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -639,38 +660,39 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
     __builtin_amdgcn_s_setprio(0);
   };
 
-  // ---- two-deep ring: tile t lives in buffer t & 1 ----------------------------------
+  // ---- two-deep ring: tile t lives in buffer (t - t_begin) & 1 -----------------------
   // Full tiles run in the loop without any masking code.  In plain mode the one partial tile (the
   // tail of the key range) is peeled off behind the loop; with query-side relocation the shared
   // range may end in a partial tile in the middle, so every tile takes the masked form there.
   constexpr bool PEEL_TAIL = MODE == MODE_PLAIN;
-  const int n_loop = PEEL_TAIL ? kv_len / BN : n_tiles;  // tiles handled inside the loop
-  load_slots(0, slot_a);
-  issue(0, lds_k0, lds_v0, slot_a);
-  load_slots(1, slot_b);
-  for (int t = 0; t < n_loop; t += 2) {
-    // even tile: wait for its copies, publish it, start the odd tile, compute
+  const int n_full = kv_len / BN;
+  const int t_stop = PEEL_TAIL ? (t_end < n_full ? t_end : n_full) : t_end;  // tiles handled inside the loop
+  load_slots(t_begin, slot_a);
+  issue(t_begin, lds_k0, lds_v0, slot_a);
+  load_slots(t_begin + 1, slot_b);
+  for (int t = t_begin; t < t_stop; t += 2) {
+    // first tile of the pair: wait for its copies, publish it, start the second, compute
     __builtin_amdgcn_s_waitcnt(0);  // this wave's copies of tile t have landed
     __syncthreads();                // ... and everybody else's; buffer 1 is no longer being read
     bool stepped = false;
-    if (t + 1 < n_tiles) {
+    if (t + 1 < t_end) {
       load_slots(t + 2, slot_a);    // slot loads go first: vmcnt retires in order, so waiting
       stepped = all_present(t + 1, slot_b);  // for them later never waits for the copies behind them
       if (!stepped) issue_slow(t + 1, lds_k1, lds_v1, slot_b);
     }
     if (nq_valid > 0) {
-      if (MODE == MODE_QUERY_SIDE && t == tiles_a && t > 0) load_q(false);  // shared keys done: back to q
+      if (MODE == MODE_QUERY_SIDE && t == tiles_a && t > t_begin) load_q(false);  // shared keys done: back to q
       const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
       compute.template operator()<!PEEL_TAIL>(lds_k0, lds_v0, tr.n_end - tr.n0, stepped, lds_k1, lds_v1, slot_b);
     } else if (stepped) {
 #pragma unroll
       for (int i = 0; i < NI; ++i) issue_rows(i, lds_k1, lds_v1, slot_b);
     }
-    if (t + 1 >= n_loop) break;
+    if (t + 1 >= t_stop) break;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     stepped = false;
-    if (t + 2 < n_tiles) {
+    if (t + 2 < t_end) {
       load_slots(t + 3, slot_b);
       stepped = all_present(t + 2, slot_a);
       if (!stepped) issue_slow(t + 2, lds_k0, lds_v0, slot_a);
@@ -684,23 +706,83 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
       for (int i = 0; i < NI; ++i) issue_rows(i, lds_k0, lds_v0, slot_a);
     }
   }
-  if (PEEL_TAIL && n_loop < n_tiles) {  // tail tile n_loop: its copies were issued one step earlier
+  if (PEEL_TAIL && t_stop < t_end) {  // tail tile t_stop: its copies were issued one step earlier
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    const bool odd = ((t_stop - t_begin) & 1) != 0;
     if (nq_valid > 0)
-      compute.template operator()<true>((n_loop & 1) ? lds_k1 : lds_k0, (n_loop & 1) ? lds_v1 : lds_v0,
-                                        kv_len - n_loop * BN, false, nullptr, nullptr, slot_a);
+      compute.template operator()<true>(odd ? lds_k1 : lds_k0, odd ? lds_v1 : lds_v0, kv_len - t_stop * BN, false,
+                                        nullptr, nullptr, slot_a);
+  }
+  __syncthreads();  // every wave is done reading the K/V ring
+
+  // ---- a unit dealt to several workgroups: leave the partial state, the last one to arrive merges ------
+  if (nparts > 1) {
+    const int my_gid = first_gid + part;
+    char *slot = p.ws_slots + (int64_t)(2 * my_gid + (part == 0 ? 1 : 0)) * kSkSlotBytes;
+    if (!(p.debug & 4))
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        *reinterpret_cast<f32x4 *>(slot + ((qt * DT + dt) * THREADS + tid) * 16) = o_acc[qt][dt];
+    float *ml = reinterpret_cast<float *>(slot + kSkAccBytes);
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) {
+      ml[(2 * qt) * THREADS + tid] = m_run[qt];
+      ml[(2 * qt + 1) * THREADS + tid] = l_acc[qt][0];
+    }
+    if (!(p.debug & 1)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // the partial state is visible device-wide ...
+    __syncthreads();
+    if (tid == 0)                                        // ... before this part counts as arrived
+      *lds_flag = __hip_atomic_fetch_add(p.ws_counters + first_gid, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*lds_flag != nparts - 1) return;  // another part is still at work: it will finish the unit
+    if (tid == 0) __hip_atomic_store(p.ws_counters + first_gid, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // Merge in part order from the slots (this part's own included, so the sum has one fixed order whoever
+    // arrives last).  The acquire fence drops what this XCD's L2 may still hold of the slots from earlier calls.
+    if (!(p.debug & 2)) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (p.debug & 8) return;
+    float m_fin[NQ16], l_fin[NQ16];
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) { m_fin[qt] = -INFINITY; l_fin[qt] = 0.0f; }
+    for (int pp = 0; pp < nparts; ++pp) {
+      const float *mlp = reinterpret_cast<const float *>(
+          p.ws_slots + (int64_t)(2 * (first_gid + pp) + (pp == 0 ? 1 : 0)) * kSkSlotBytes + kSkAccBytes);
+#pragma unroll
+      for (int qt = 0; qt < NQ16; ++qt) m_fin[qt] = fmaxf(m_fin[qt], mlp[(2 * qt) * THREADS + tid]);
+    }
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = f32x4{0, 0, 0, 0};
+    for (int pp = 0; pp < nparts; ++pp) {
+      const char *src = p.ws_slots + (int64_t)(2 * (first_gid + pp) + (pp == 0 ? 1 : 0)) * kSkSlotBytes;
+      const float *mlp = reinterpret_cast<const float *>(src + kSkAccBytes);
+#pragma unroll
+      for (int qt = 0; qt < NQ16; ++qt) {
+        const float mp = mlp[(2 * qt) * THREADS + tid];
+        const float lp = mlp[(2 * qt + 1) * THREADS + tid];
+        const float a = mp == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mp - m_fin[qt]);
+        l_fin[qt] += lp * a;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          o_acc[qt][dt] += *reinterpret_cast<const f32x4 *>(src + ((qt * DT + dt) * THREADS + tid) * 16) * a;
+      }
+    }
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) l_acc[qt][0] = l_fin[qt];
   }
 
   // ---- epilogue: normalise, transpose through LDS, store whole 16-byte chunks ------------------
   // Lane layout of O^T (query li, features 16*dt + 4*lg .. +4) would give 8-byte stores scattered
   // over 16 rows; staging the wave's WQ x D tile in LDS (one 16 KiB ring buffer per wave, rows padded
   // to 272 B against bank conflicts) lets 16 consecutive lanes write one full output row.
-  __syncthreads();  // every wave is done reading the K/V ring
   {
     constexpr int OPITCH = ROW_BYTES + 16;
-    static_assert(WQ * OPITCH <= TILE_BYTES, "per-wave output staging must fit one ring buffer");
-    char *stage = wave == 0 ? lds_k0 : wave == 1 ? lds_v0 : wave == 2 ? lds_k1 : lds_v1;
+    // the four ring buffers are one block; the callers make it at least NW * WQ * OPITCH bytes
+    static_assert(NW != 4 || WQ * OPITCH <= TILE_BYTES, "per-wave output staging must fit one ring buffer");
+    char *stage = lds_k0 + wave * (NW == 4 ? TILE_BYTES : WQ * OPITCH);
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt) {
       const float l = l_acc[qt][0];
@@ -727,17 +809,30 @@ __device__ __forceinline__ void attn_dma_tile(const AttnParams &p, char *lds_k0,
   }
 }
 
-template <int DTYPE, int D, int NQ16, int MODE>
-__global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
-  static_assert(MODE != MODE_KEY_SIDE, "key-side rotation needs the register-staged kernel");
-  constexpr int BM = 64 * NQ16;               // query rows per tile
+// Key tiles of request b as attn_dma_part walks them (query-side mode: the shared range and the rest are tiled
+// separately); a request without keys keeps one virtual tile so that somebody owns its (zero) output rows.
+template <int MODE>
+__device__ __forceinline__ int sk_key_tiles(const AttnParams &p, int b, int kv_len) {
+  if (kv_len <= 0) return 1;
+  if (MODE != MODE_QUERY_SIDE) return (kv_len + 63) / 64;
+  int shared = p.shared_kv_lens[b];
+  shared = shared < 0 ? 0 : (shared > kv_len ? kv_len : shared);
+  return (shared + 63) / 64 + (kv_len - shared + 63) / 64;
+}
+
+// One workgroup per unit, units dealt whole: blocks are handed out in index order, which with the
+// longest-request-first tile order of locate_query_tile_lpt is longest-processing-time-first list scheduling.
+template <int DTYPE, int D, int MODE, int NW = 4>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_kernel(AttnParams p) {
+  constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = 64 * D * 2;
-
-  __shared__ __attribute__((aligned(16))) char lds_k0[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char lds_v0[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char lds_k1[TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char lds_v1[TILE_BYTES];
-
+  constexpr int STAGING = NW * 32 * (D * 2 + 16);
+  // one block, so that the ring keeps its 1 KiB alignment (the swizzle that makes the fragment reads
+  // conflict-free counts on it) and the flag word sits behind it
+  __shared__ __attribute__((aligned(1024))) char lds[(4 * TILE_BYTES > STAGING ? 4 * TILE_BYTES : STAGING) + 16];
+  char *const lds_k0 = lds, *const lds_v0 = lds + TILE_BYTES;
+  char *const lds_k1 = lds + 2 * TILE_BYTES, *const lds_v1 = lds + 3 * TILE_BYTES;
+  int &lds_flag = *reinterpret_cast<int *>(lds + (4 * TILE_BYTES > STAGING ? 4 * TILE_BYTES : STAGING));
   int tile, kvh, hg;
   if (!block_to_tile_head(p, tile, kvh, hg)) return;
   const int group = p.H / p.H_kv;
@@ -750,38 +845,41 @@ __global__ __launch_bounds__(256, 2) void varlen_attn_dma_kernel(AttnParams p) {
     if (!found) return;
     tile = tile_in_request;
   }
-
-  // The last query tile of a request may hold few rows.  With at most half a tile left the four waves take
-  // 16 rows each instead of 32: the workgroup streams the same K/V but with half the matrix and softmax work per
-  // wave, and finishes in about two thirds of the time.
   const int q_tile0 = tile * BM;
-  if (NQ16 == 2 && q_len - q_tile0 <= BM / 2)
-    attn_dma_tile<DTYPE, D, 1, MODE>(p, lds_k0, lds_v0, lds_k1, lds_v1, b, q_begin, q_len, q_tile0, head, kvh);
+  const int kt = sk_key_tiles<MODE>(p, b, p.cu_k[b + 1] - p.cu_k[b]);
+  if (q_len - q_tile0 <= BM / 2)
+    attn_dma_part<DTYPE, D, 1, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, &lds_flag, b, q_begin, q_len, q_tile0, head,
+                                         kvh, 0, kt, 1, 0, 0);
   else
-    attn_dma_tile<DTYPE, D, NQ16, MODE>(p, lds_k0, lds_v0, lds_k1, lds_v1, b, q_begin, q_len, q_tile0, head, kvh);
+    attn_dma_part<DTYPE, D, 2, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, &lds_flag, b, q_begin, q_len, q_tile0, head,
+                                         kvh, 0, kt, 1, 0, 0);
 }
 
 template <int DTYPE, int D, int NQ16>
-static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStream_t stream) {
+static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, void *workspace, int64_t workspace_bytes,
+                       hipStream_t stream) {
   AttnParams p = p0;
-  constexpr int BM = 64 * NQ16;
-  p.num_tiles = (int32_t)((total_q + BM - 1) / BM) + p.B;
-  int64_t blocks = ((int64_t)p.num_tiles * p.H + 7) / 8 * 8;  // the register-staged kernel's own linear mapping
-  if (mode != MODE_KEY_SIDE) blocks = attn_grid_blocks(p);
-  if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
-  dim3 grid((unsigned)blocks), block(256);
-  switch (mode) {
-    case MODE_PLAIN:
-      hipLaunchKernelGGL((varlen_attn_dma_kernel<DTYPE, D, NQ16, MODE_PLAIN>), grid, block, 0, stream, p);
-      break;
-    case MODE_KEY_SIDE:
-      hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_KEY_SIDE>), grid, block, 0, stream, p);
-      break;
-    default:
-      hipLaunchKernelGGL((varlen_attn_dma_kernel<DTYPE, D, NQ16, MODE_QUERY_SIDE>), grid, block, 0, stream, p);
-      break;
+  if (mode == MODE_KEY_SIDE) {
+    constexpr int BM = 64 * NQ16;
+    p.num_tiles = (int32_t)((total_q + BM - 1) / BM) + p.B;
+    const int64_t blocks = ((int64_t)p.num_tiles * p.H + 7) / 8 * 8;  // the register-staged kernel's own linear mapping
+    if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
+    hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_KEY_SIDE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    return launch_status("varlen_attn_kernel");
   }
-  return launch_status("varlen_attn_kernel");
+  { const char *dbg = getenv("ACACHE_SK_DEBUG"); p.debug = dbg ? atoi(dbg) : 0; }
+  // More than 128 query rows per request on average: 8-wave workgroups that own up to 256 rows of a head, on a
+  // persistent grid.  Otherwise one 4-wave workgroup per (request, 128-row query tile, head).
+  if (total_q > (int64_t)128 * p.B && (p.debug & 32))  // work in progress: opt-in while the wide kernel is tuned
+    return launch_attn_wide(p, DTYPE, D, mode, (p.debug & 1) ? nullptr : workspace, workspace_bytes, stream);
+  p.num_tiles = (int32_t)((total_q + 127) / 128) + p.B;
+  const int64_t blocks = attn_grid_blocks(p);
+  if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
+  if (mode == MODE_PLAIN)
+    hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_PLAIN>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  else
+    hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_QUERY_SIDE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  return launch_status("varlen_attn_unit_kernel");
 }
 
 // Any other head_dim (a multiple of 16 up to 256): the register-staged kernel at a padded width of 256,
@@ -814,6 +912,8 @@ static int launch_attn_any_head_dim(const AttnParams &p0, int mode, int64_t tota
 
 using namespace acache;
 
+extern "C" int64_t acache_varlen_attn_workspace_bytes(void) { return attn_wide_workspace_bytes(); }
+
 extern "C" int acache_varlen_attn(
     void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *cu_q,
     const int32_t *cu_k, const int32_t *slot_map, float scale, int32_t shared_prefix_len,
@@ -821,7 +921,7 @@ extern "C" int acache_varlen_attn(
     const float *rope_sin, int32_t rope_rows, int32_t B, int64_t total_q, int64_t total_k, int32_t H,
     int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t q_token_stride,
     int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t kv_slot_stride,
-    int64_t kv_head_stride, void *stream) {
+    int64_t kv_head_stride, void *workspace, int64_t workspace_bytes, void *stream) {
   if (dtype != ACACHE_BF16 && dtype != ACACHE_F16)
     return fail(ACACHE_E_DTYPE, "varlen_attn: dtype %d not supported (bf16 or f16)", dtype);
   if (D < 16 || D > 256 || D % 16 != 0)
@@ -839,6 +939,8 @@ extern "C" int acache_varlen_attn(
   if (relocate && (!rope_cos || !rope_sin || rope_rows <= 0))
     return fail(ACACHE_E_MODE, "varlen_attn: relocation requested without RoPE tables");
   const int es = 2;
+  if (workspace_bytes < 0 || (workspace && !aligned16(workspace)))
+    return fail(ACACHE_E_ALIGN, "varlen_attn: workspace must be 16-byte aligned, its size non-negative");
   if (!aligned16(out) || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) ||
       (q_token_stride * es) % 16 || (q_head_stride * es) % 16 || (out_token_stride * es) % 16 ||
       (out_head_stride * es) % 16 || (kv_slot_stride * es) % 16 || (kv_head_stride * es) % 16)
@@ -856,10 +958,11 @@ extern "C" int acache_varlen_attn(
   p.q_token_bytes = q_token_stride * es; p.q_head_bytes = q_head_stride * es;
   p.o_token_bytes = out_token_stride * es; p.o_head_bytes = out_head_stride * es;
   p.kv_slot_bytes = kv_slot_stride * es; p.kv_head_bytes = kv_head_stride * es;
+  p.ws_slots = nullptr; p.ws_counters = nullptr; p.debug = 0;
   const int mode = query_side ? MODE_QUERY_SIDE : (relocate ? MODE_KEY_SIDE : MODE_PLAIN);
   hipStream_t st = (hipStream_t)stream;
 #define ACACHE_ATTN(DT, DD) \
-  if (dtype == DT && D == DD) return launch_attn<DT, DD, 2>(p, mode, total_q, st);
+  if (dtype == DT && D == DD) return launch_attn<DT, DD, 2>(p, mode, total_q, workspace, workspace_bytes, st);
   ACACHE_ATTN(ACACHE_BF16, 128)
   ACACHE_ATTN(ACACHE_BF16, 64)
   ACACHE_ATTN(ACACHE_F16, 128)

@@ -38,6 +38,11 @@ struct AttnParams {
   int64_t q_token_bytes, q_head_bytes;
   int64_t o_token_bytes, o_head_bytes;
   int64_t kv_slot_bytes, kv_head_bytes;
+  // persistent schedule: partial-state slots and arrival counters of units dealt to several workgroups
+  // (NULL: units are never split)
+  char *ws_slots;
+  int32_t *ws_counters;
+  int32_t debug;
 };
 
 // Which (request, query tile) does global tile index `tile` address?  Lane i loads
@@ -118,9 +123,16 @@ __device__ __forceinline__ bool block_to_tile_head(const AttnParams &p, int &til
   const int group = p.H / p.H_kv;
   if (p.H_kv % 8 == 0) {
     const int heads_per_xcd = (p.H_kv >> 3) * group;
+    int r;
+    if (p.debug & 2048) {  // heads outermost: all query tiles of one head before the next head
+      r = idx / p.num_tiles;
+      if (r >= heads_per_xcd) return false;
+      tile = idx - r * p.num_tiles;
+    } else {
     tile = idx / heads_per_xcd;
     if (tile >= p.num_tiles) return false;
-    const int r = idx - tile * heads_per_xcd;
+    r = idx - tile * heads_per_xcd;
+    }
     kvh = xcd * (p.H_kv >> 3) + r / group;
     hg = r % group;
   } else if (8 % p.H_kv == 0) {
@@ -187,12 +199,14 @@ __device__ __forceinline__ void lds_dma16(const char *src, char *lds_dst) {
 //          query's maximum jumped by more than 8 — one wave-uniform test per tile of 16 queries,
 //          rarely true after the first key tile.
 //   MASKED keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
-template <int NQ16, int NT, int DT, bool MASKED>
+//   NQA    the first NQA of the wave's NQ16 query tiles are live; the others are left alone
+template <int NQA, int NQ16, int NT, int DT, bool MASKED>
 __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], float (&m_run)[NQ16],
                                                   f32x4 (&l_acc)[NQ16], f32x4 (&o_acc)[NQ16][DT],
                                                   float c, int n_valid, int lg) {
+  static_assert(NQA <= NQ16, "live query tiles");
 #pragma unroll
-  for (int qt = 0; qt < NQ16; ++qt) {
+  for (int qt = 0; qt < NQA; ++qt) {
     if (MASKED && n_valid < 16 * NT) {  // wave-uniform: full tiles skip the masking code
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
@@ -227,12 +241,12 @@ __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], floa
 // l_acc is accumulated by the matrix core as one more row block of O^T whose V^T rows are all
 // ones: every element of l_acc[qt] ends up holding sum_n P[n][query li] of the ROUNDED
 // probabilities, with no VALU adds or cross-lane reduction.  Slabs must be taken in order.
-template <class M, int S, int NQ16, int NT, int NS>
+template <class M, int S, int NQA, int NQ16, int NT, int NS>
 __device__ __forceinline__ void softmax_probs_slab(const f32x4 (&s_acc)[NQ16][NT], const float (&m_run)[NQ16],
                                                    f32x4 (&l_acc)[NQ16], vec16 (&pf)[NQ16][NS],
                                                    const vec16 &ones, float c) {
 #pragma unroll
-  for (int qt = 0; qt < NQ16; ++qt) {
+  for (int qt = 0; qt < NQA; ++qt) {
     const float mc = m_run[qt];
     float e[8];
 #pragma unroll
@@ -244,5 +258,10 @@ __device__ __forceinline__ void softmax_probs_slab(const f32x4 (&s_acc)[NQ16][NT
     l_acc[qt] = M::run(ones, pf[qt][S], l_acc[qt]);
   }
 }
+
+// 8-wave persistent kernel for requests with more than 128 query rows (attn_wide.hip)
+int64_t attn_wide_workspace_bytes();
+int launch_attn_wide(const AttnParams &p, int dtype, int D, int mode, void *workspace, int64_t workspace_bytes,
+                     hipStream_t stream);
 
 }  // namespace acache

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define ACACHE_ABI_VERSION 1
+#define ACACHE_ABI_VERSION 2
 
 /* element types of K/V/Q payloads */
 #define ACACHE_BF16 0
@@ -343,7 +343,20 @@ int acache_build_slot_layout(
  * slot lies outside [0, num_slots) reads as a zero row.
  * q / out: [total_q, H, D] with given token and head strides (innermost 1).
  * k_cache / v_cache: [num_slots, H_kv, D] with given slot and head strides.
+ *
+ * Schedule and workspace (head_dim 64 / 128, plain and query-side modes).  The kernel is launched as
+ * a persistent grid of two workgroups per CU; the (request, 128-row query tile, head) units are laid
+ * end to end and every workgroup takes an equal share of key-tile steps, so a unit may be cut between
+ * neighbouring workgroups.  The parts of a cut unit meet in `workspace`: device memory of at least
+ * acache_varlen_attn_workspace_bytes() bytes (a function of the current device's CU count: arrival
+ * counters followed by two partial-state slots per workgroup), 16-byte aligned, owned by the caller.
+ * Its counters must be ZERO before the first call that uses it (clear the buffer once after
+ * allocating it); every call leaves them zero again, so the buffer is reusable as is.  Calls that
+ * may overlap in time (different streams) need different workspaces.  The merge order is fixed, so
+ * results are bit-identical from run to run.  workspace == NULL (or smaller than required): units are
+ * never cut and are dealt whole instead — same results up to the rounding of the merge, longer tail.
  */
+int64_t acache_varlen_attn_workspace_bytes(void);
 int acache_varlen_attn(
     void *out, const void *q, const void *k_cache, const void *v_cache,
     const int32_t *cu_q, const int32_t *cu_k, const int32_t *slot_map,
@@ -355,7 +368,7 @@ int acache_varlen_attn(
     int64_t q_token_stride, int64_t q_head_stride,
     int64_t out_token_stride, int64_t out_head_stride,
     int64_t kv_slot_stride, int64_t kv_head_stride,
-    void *stream);
+    void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
  * Two elementwise steps of the decoder block on either side of the attention path, for
