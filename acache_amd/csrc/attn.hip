@@ -384,26 +384,12 @@ __global__ __launch_bounds__(256, RAGGED ? 1 : 2) void varlen_attn_kernel(AttnPa
 // 4*j + i/4, j = 0..3.  With lane l pointing at V[row0 + l/4][d0 + 4*(l%4)] lane i
 // gets V[row0 + 0..3][d0 + i]: four keys of one column, i.e. half of an MFMA
 // A-operand of V^T.
-// Partial results of a (query tile, head) unit whose key tiles were dealt to several workgroups: every
-// part leaves its un-normalised O^T accumulators, running reference m and running sum l in its workspace
-// slot, in register order (thread-major, 16 bytes per thread and register quad, so the stores coalesce).
-constexpr int kSkThreads = 256;
-constexpr int kSkAccBytes = kSkThreads * 16 * 16;            // 2 query tiles x 8 d tiles x 16 B per thread
-constexpr int kSkSlotBytes = kSkAccBytes + kSkThreads * 4 * 4;  // + (m, l) of the two query tiles
-constexpr int kSkCounterAlign = 4096;
-
-// Key tiles [t_begin, t_end) of one query tile of one (request, head): the four waves take WQ = 16 * NQ16 query
-// rows each, starting at row q_tile0 of the request, and stream the tiles through the LDS ring.
-// nparts == 1: the range is the whole unit and the result goes to `out`.  nparts > 1: the unit's tiles were dealt
-// to nparts consecutive workgroups (this one holds part `part`, the first one has global index first_gid); every
-// part writes its partial state to its workspace slot and bumps the unit's counter, and the part that finds
-// all the others already there merges them in part order (so the result does not depend on arrival order),
-// resets the counter and writes `out`.  Nobody waits for anybody.
+// One query tile of one (request, head): the NW waves take WQ = 16 * NQ16 query rows each, starting at row
+// q_tile0 of the request, and stream the request's key tiles [t_begin, t_end) through the LDS ring.
 template <int DTYPE, int D, int NQ16, int MODE, int NW = 4>
 __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0, char *lds_v0, char *lds_k1,
-                                              char *lds_v1, int *lds_flag, int b, int q_begin, int q_len,
-                                              int q_tile0, int head, int kvh, int t_begin, int t_end, int nparts,
-                                              int part, int first_gid) {
+                                              char *lds_v1, float *lds_rope, int b, int q_begin, int q_len, int q_tile0,
+                                              int head, int kvh, int t_begin, int t_end) {
   constexpr int BN = 64;
   constexpr int WQ = 16 * NQ16;
   constexpr int KS = D / 32;
@@ -433,9 +419,6 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   int nq_valid = (q_len - q_wave0 + 15) / 16;
   nq_valid = nq_valid < 0 ? 0 : (nq_valid > NQ16 ? NQ16 : nq_valid);
   char *out_base = p.out + (int64_t)q_begin * p.o_token_bytes + (int64_t)head * p.o_head_bytes;
-
-  // the previous unit of this workgroup may still be reading the ring (its output staging) and the flag word
-  __syncthreads();
 
   if (kv_len <= 0) {
     for (int r = tid / CH; r < NW * WQ; r += THREADS / CH) {
@@ -660,11 +643,62 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     __builtin_amdgcn_s_setprio(0);
   };
 
+  // Key-side relocation: the rows of tile t whose slot lies in the shared range are re-rotated in place, in
+  // LDS, right after the tile has landed — once per workgroup and key tile, with the arithmetic of the
+  // stand-alone relocation kernel (products and sum rounded separately, one rounding to the cache type), so
+  // attention over the rotated tile equals attention over a materialised copy bit for bit.  Thread -> (row
+  // tid / 4, a quarter of the row's chunk pairs); chunk c of row r sits at chunk position c ^ f_K(r).
+  // Every shared row has its own shift n - slot; in the engine's layouts all shared rows of a request have the
+  // shift the caller also passes per request, so the cos / sin rows of that shift are kept in LDS (lds_rope,
+  // filled below) and only rows with another shift fetch their own rows from the table.  The row's slot is
+  // fetched one tile ahead (rot_slot), behind the compute phase of the tile before.
+  constexpr int PAIRS = CH / 2;                    // (d, d + D/2) chunk pairs per row
+  constexpr int PER_THREAD = BN * PAIRS / THREADS;  // 2 (D = 128, 4 waves)
+  static_assert(BN * PAIRS % THREADS == 0 && PER_THREAD >= 1, "one or more chunk pairs per thread");
+  const int rot_row = tid / (PAIRS / PER_THREAD);
+  int shift0 = 0;
+  if (MODE == MODE_KEY_SIDE) {
+    shift0 = p.affix_shifts[b];
+    if (shift0 < 0 || shift0 >= p.rope_rows) shift0 = 0;
+    if (tid < 2 * D / 4) {  // cos row, then sin row: D floats each, 16 bytes per thread
+      const float *src = (tid < D / 4 ? p.cos_tab : p.sin_tab) + (int64_t)shift0 * D + (tid % (D / 4)) * 4;
+      store16(lds_rope + tid * 4, load16(src));
+    }  // published by the barrier that publishes the first tile
+  }
+  auto rot_prefetch = [&](int t) __attribute__((always_inline)) {
+    const int n = t * BN + rot_row;
+    return MODE == MODE_KEY_SIDE && t < t_end && n < kv_len ? p.slot_map[kv_begin + n] : -1;
+  };
+  auto rotate_shared_rows = [&](char *kbuf, int t, int slot) __attribute__((always_inline)) {
+    const int n = t * BN + rot_row;
+    const int delta = n - slot;
+    const int ad = delta < 0 ? -delta : delta;
+    if (n < kv_len && slot >= 0 && slot < p.shared_prefix_len && delta != 0 && ad < p.rope_rows) {
+      char *row = kbuf + rot_row * ROW_BYTES;
+      const int f = (rot_row / RW) % CH;
+      auto rotate_with = [&](const float *cr, const float *sr) __attribute__((always_inline)) {
+#pragma unroll
+        for (int k = 0; k < PER_THREAD; ++k) {
+          const int c = (tid % (PAIRS / PER_THREAD)) * PER_THREAD + k;
+          char *lo_p = row + ((c ^ f) << 4), *hi_p = row + (((c + PAIRS) ^ f) << 4);
+          vec16 lo = load16(lo_p), hi = load16(hi_p);
+          rotate_pair_half_fast<DTYPE>(lo, hi, cr, sr, c * 8, D / 2, delta < 0 ? -1.0f : 1.0f);
+          store16(lo_p, lo);
+          store16(hi_p, hi);
+        }
+      };
+      if (delta == shift0) rotate_with(lds_rope, lds_rope + D);  // separate calls: LDS reads here, global loads there
+      else rotate_with(p.cos_tab + (int64_t)ad * D, p.sin_tab + (int64_t)ad * D);
+    }
+    __syncthreads();  // the rotated rows are in place for everybody
+  };
+  int rot_slot = rot_prefetch(t_begin);
+
   // ---- two-deep ring: tile t lives in buffer (t - t_begin) & 1 -----------------------
   // Full tiles run in the loop without any masking code.  In plain mode the one partial tile (the
   // tail of the key range) is peeled off behind the loop; with query-side relocation the shared
   // range may end in a partial tile in the middle, so every tile takes the masked form there.
-  constexpr bool PEEL_TAIL = MODE == MODE_PLAIN;
+  constexpr bool PEEL_TAIL = MODE != MODE_QUERY_SIDE;
   const int n_full = kv_len / BN;
   const int t_stop = PEEL_TAIL ? (t_end < n_full ? t_end : n_full) : t_end;  // tiles handled inside the loop
   load_slots(t_begin, slot_a);
@@ -674,6 +708,11 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     // first tile of the pair: wait for its copies, publish it, start the second, compute
     __builtin_amdgcn_s_waitcnt(0);  // this wave's copies of tile t have landed
     __syncthreads();                // ... and everybody else's; buffer 1 is no longer being read
+    if (MODE == MODE_KEY_SIDE) {
+      const int cur = rot_slot;
+      rot_slot = rot_prefetch(t + 1);
+      rotate_shared_rows(lds_k0, t, cur);
+    }
     bool stepped = false;
     if (t + 1 < t_end) {
       load_slots(t + 2, slot_a);    // slot loads go first: vmcnt retires in order, so waiting
@@ -691,6 +730,11 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     if (t + 1 >= t_stop) break;
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    if (MODE == MODE_KEY_SIDE) {
+      const int cur = rot_slot;
+      rot_slot = rot_prefetch(t + 2);
+      rotate_shared_rows(lds_k1, t + 1, cur);
+    }
     stepped = false;
     if (t + 2 < t_end) {
       load_slots(t + 3, slot_b);
@@ -710,69 +754,12 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     const bool odd = ((t_stop - t_begin) & 1) != 0;
+    if (MODE == MODE_KEY_SIDE) rotate_shared_rows(odd ? lds_k1 : lds_k0, t_stop, rot_slot);
     if (nq_valid > 0)
       compute.template operator()<true>(odd ? lds_k1 : lds_k0, odd ? lds_v1 : lds_v0, kv_len - t_stop * BN, false,
                                         nullptr, nullptr, slot_a);
   }
   __syncthreads();  // every wave is done reading the K/V ring
-
-  // ---- a unit dealt to several workgroups: leave the partial state, the last one to arrive merges ------
-  if (nparts > 1) {
-    const int my_gid = first_gid + part;
-    char *slot = p.ws_slots + (int64_t)(2 * my_gid + (part == 0 ? 1 : 0)) * kSkSlotBytes;
-    if (!(p.debug & 4))
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt)
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt)
-        *reinterpret_cast<f32x4 *>(slot + ((qt * DT + dt) * THREADS + tid) * 16) = o_acc[qt][dt];
-    float *ml = reinterpret_cast<float *>(slot + kSkAccBytes);
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt) {
-      ml[(2 * qt) * THREADS + tid] = m_run[qt];
-      ml[(2 * qt + 1) * THREADS + tid] = l_acc[qt][0];
-    }
-    if (!(p.debug & 1)) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // the partial state is visible device-wide ...
-    __syncthreads();
-    if (tid == 0)                                        // ... before this part counts as arrived
-      *lds_flag = __hip_atomic_fetch_add(p.ws_counters + first_gid, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (*lds_flag != nparts - 1) return;  // another part is still at work: it will finish the unit
-    if (tid == 0) __hip_atomic_store(p.ws_counters + first_gid, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // Merge in part order from the slots (this part's own included, so the sum has one fixed order whoever
-    // arrives last).  The acquire fence drops what this XCD's L2 may still hold of the slots from earlier calls.
-    if (!(p.debug & 2)) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    if (p.debug & 8) return;
-    float m_fin[NQ16], l_fin[NQ16];
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt) { m_fin[qt] = -INFINITY; l_fin[qt] = 0.0f; }
-    for (int pp = 0; pp < nparts; ++pp) {
-      const float *mlp = reinterpret_cast<const float *>(
-          p.ws_slots + (int64_t)(2 * (first_gid + pp) + (pp == 0 ? 1 : 0)) * kSkSlotBytes + kSkAccBytes);
-#pragma unroll
-      for (int qt = 0; qt < NQ16; ++qt) m_fin[qt] = fmaxf(m_fin[qt], mlp[(2 * qt) * THREADS + tid]);
-    }
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt)
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = f32x4{0, 0, 0, 0};
-    for (int pp = 0; pp < nparts; ++pp) {
-      const char *src = p.ws_slots + (int64_t)(2 * (first_gid + pp) + (pp == 0 ? 1 : 0)) * kSkSlotBytes;
-      const float *mlp = reinterpret_cast<const float *>(src + kSkAccBytes);
-#pragma unroll
-      for (int qt = 0; qt < NQ16; ++qt) {
-        const float mp = mlp[(2 * qt) * THREADS + tid];
-        const float lp = mlp[(2 * qt + 1) * THREADS + tid];
-        const float a = mp == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mp - m_fin[qt]);
-        l_fin[qt] += lp * a;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-          o_acc[qt][dt] += *reinterpret_cast<const f32x4 *>(src + ((qt * DT + dt) * THREADS + tid) * 16) * a;
-      }
-    }
-#pragma unroll
-    for (int qt = 0; qt < NQ16; ++qt) l_acc[qt][0] = l_fin[qt];
-  }
 
   // ---- epilogue: normalise, transpose through LDS, store whole 16-byte chunks ------------------
   // Lane layout of O^T (query li, features 16*dt + 4*lg .. +4) would give 8-byte stores scattered
@@ -828,11 +815,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
   constexpr int TILE_BYTES = 64 * D * 2;
   constexpr int STAGING = NW * 32 * (D * 2 + 16);
   // one block, so that the ring keeps its 1 KiB alignment (the swizzle that makes the fragment reads
-  // conflict-free counts on it) and the flag word sits behind it
-  __shared__ __attribute__((aligned(1024))) char lds[(4 * TILE_BYTES > STAGING ? 4 * TILE_BYTES : STAGING) + 16];
+  // conflict-free counts on it)
+  // (+ the cos / sin rows of the request's shift in key-side mode)
+  __shared__ __attribute__((aligned(1024))) char lds[(4 * TILE_BYTES > STAGING ? 4 * TILE_BYTES : STAGING) +
+                                                     (MODE == MODE_KEY_SIDE ? 2 * D * 4 : 0)];
+  float *const lds_rope = reinterpret_cast<float *>(lds + (4 * TILE_BYTES > STAGING ? 4 * TILE_BYTES : STAGING));
   char *const lds_k0 = lds, *const lds_v0 = lds + TILE_BYTES;
   char *const lds_k1 = lds + 2 * TILE_BYTES, *const lds_v1 = lds + 3 * TILE_BYTES;
-  int &lds_flag = *reinterpret_cast<int *>(lds + (4 * TILE_BYTES > STAGING ? 4 * TILE_BYTES : STAGING));
   int tile, kvh, hg;
   if (!block_to_tile_head(p, tile, kvh, hg)) return;
   const int group = p.H / p.H_kv;
@@ -848,35 +837,32 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
   const int q_tile0 = tile * BM;
   const int kt = sk_key_tiles<MODE>(p, b, p.cu_k[b + 1] - p.cu_k[b]);
   if (q_len - q_tile0 <= BM / 2)
-    attn_dma_part<DTYPE, D, 1, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, &lds_flag, b, q_begin, q_len, q_tile0, head,
-                                         kvh, 0, kt, 1, 0, 0);
+    attn_dma_part<DTYPE, D, 1, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
+                                         0, kt);
   else
-    attn_dma_part<DTYPE, D, 2, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, &lds_flag, b, q_begin, q_len, q_tile0, head,
-                                         kvh, 0, kt, 1, 0, 0);
+    attn_dma_part<DTYPE, D, 2, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
+                                         0, kt);
 }
 
 template <int DTYPE, int D, int NQ16>
 static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, void *workspace, int64_t workspace_bytes,
                        hipStream_t stream) {
   AttnParams p = p0;
-  if (mode == MODE_KEY_SIDE) {
-    constexpr int BM = 64 * NQ16;
-    p.num_tiles = (int32_t)((total_q + BM - 1) / BM) + p.B;
-    const int64_t blocks = ((int64_t)p.num_tiles * p.H + 7) / 8 * 8;  // the register-staged kernel's own linear mapping
-    if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
-    hipLaunchKernelGGL((varlen_attn_kernel<DTYPE, D, NQ16, MODE_KEY_SIDE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
-    return launch_status("varlen_attn_kernel");
-  }
-  { const char *dbg = getenv("ACACHE_SK_DEBUG"); p.debug = dbg ? atoi(dbg) : 0; }
-  // More than 128 query rows per request on average: 8-wave workgroups that own up to 256 rows of a head, on a
-  // persistent grid.  Otherwise one 4-wave workgroup per (request, 128-row query tile, head).
-  if (total_q > (int64_t)128 * p.B && (p.debug & 32))  // work in progress: opt-in while the wide kernel is tuned
-    return launch_attn_wide(p, DTYPE, D, mode, (p.debug & 1) ? nullptr : workspace, workspace_bytes, stream);
+  // One 4-wave workgroup per (request, 128-row query tile, head) is the default.  The 8-wave persistent kernel
+  // (attn_wide.hip) is faster on batches of equal requests with 129 .. 256 query rows (17 - 22 % measured) and
+  // slower on ragged ones (it runs one workgroup per CU, so the start-up and wind-down of every part it is
+  // dealt are exposed instead of hidden behind a second workgroup): it is taken only when the caller asks for
+  // it with ACACHE_ATTN_WIDE=1 in the environment.
+  static const bool wide_opt_in = [] { const char *e = getenv("ACACHE_ATTN_WIDE"); return e && e[0] == '1'; }();
+  if (wide_opt_in && mode != MODE_KEY_SIDE && total_q > (int64_t)128 * p.B)
+    return launch_attn_wide(p, DTYPE, D, mode, workspace, workspace_bytes, stream);
   p.num_tiles = (int32_t)((total_q + 127) / 128) + p.B;
   const int64_t blocks = attn_grid_blocks(p);
   if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
   if (mode == MODE_PLAIN)
     hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_PLAIN>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  else if (mode == MODE_KEY_SIDE)
+    hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_KEY_SIDE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
   else
     hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_QUERY_SIDE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
   return launch_status("varlen_attn_unit_kernel");
@@ -958,7 +944,7 @@ extern "C" int acache_varlen_attn(
   p.q_token_bytes = q_token_stride * es; p.q_head_bytes = q_head_stride * es;
   p.o_token_bytes = out_token_stride * es; p.o_head_bytes = out_head_stride * es;
   p.kv_slot_bytes = kv_slot_stride * es; p.kv_head_bytes = kv_head_stride * es;
-  p.ws_slots = nullptr; p.ws_counters = nullptr; p.debug = 0;
+  p.ws_slots = nullptr; p.ws_counters = nullptr;
   const int mode = query_side ? MODE_QUERY_SIDE : (relocate ? MODE_KEY_SIDE : MODE_PLAIN);
   hipStream_t st = (hipStream_t)stream;
 #define ACACHE_ATTN(DT, DD) \

@@ -42,7 +42,6 @@ struct AttnParams {
   // (NULL: units are never split)
   char *ws_slots;
   int32_t *ws_counters;
-  int32_t debug;
 };
 
 // Which (request, query tile) does global tile index `tile` address?  Lane i loads
@@ -123,16 +122,9 @@ __device__ __forceinline__ bool block_to_tile_head(const AttnParams &p, int &til
   const int group = p.H / p.H_kv;
   if (p.H_kv % 8 == 0) {
     const int heads_per_xcd = (p.H_kv >> 3) * group;
-    int r;
-    if (p.debug & 2048) {  // heads outermost: all query tiles of one head before the next head
-      r = idx / p.num_tiles;
-      if (r >= heads_per_xcd) return false;
-      tile = idx - r * p.num_tiles;
-    } else {
     tile = idx / heads_per_xcd;
     if (tile >= p.num_tiles) return false;
-    r = idx - tile * heads_per_xcd;
-    }
+    const int r = idx - tile * heads_per_xcd;
     kvh = xcd * (p.H_kv >> 3) + r / group;
     hg = r % group;
   } else if (8 % p.H_kv == 0) {
@@ -208,11 +200,12 @@ __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], floa
 #pragma unroll
   for (int qt = 0; qt < NQA; ++qt) {
     if (MASKED && n_valid < 16 * NT) {  // wave-uniform: full tiles skip the masking code
+      const int limit = n_valid - 4 * lg;  // one lane-dependent value; the row offsets below are immediates
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (16 * nt + 4 * lg + i >= n_valid) s_acc[qt][nt][i] = -INFINITY;
+          if (16 * nt + i >= limit) s_acc[qt][nt][i] = -INFINITY;
     }
     float mx = -INFINITY;
 #pragma unroll

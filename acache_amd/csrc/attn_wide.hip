@@ -35,7 +35,7 @@ constexpr int kWideTableTiles = 64;              // key tiles whose slots the LD
 // partial state of one part: 16 accumulator quads + (m, l) of the two query tiles, per thread, thread-major
 constexpr int kWideAccBytes = kWideThreads * 16 * 16;
 constexpr int kWideSlotBytes = kWideAccBytes + kWideThreads * 4 * 4;
-constexpr int kWideCounterAlign = 131072;  // DEBUG: room for time stamps
+constexpr int kWideCounterAlign = 4096;
 
 // ---- the timeline ------------------------------------------------------------------------------------------
 // Weights in twentieths of a full key-tile step.  A unit weighs kUnit + tiles * c, c by the busiest SIMD's
@@ -586,7 +586,6 @@ __global__ __launch_bounds__(kWideThreads, 1) void varlen_attn_wide_kernel(AttnP
   // computed only a loop counter is live.  Kept alive across the key loop they push it over the scalar-register
   // budget, and the instruction scheduler answers excess pressure by giving up the early issue of the fragment
   // reads that the loop depends on.)
-  const unsigned long long t_entry = wall_clock64();
   if (threadIdx.x < 64) {  // wave 0 lays the workgroup's stretch out; everybody reads it from LDS
     const int lane = threadIdx.x;
     const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
@@ -733,17 +732,8 @@ __global__ __launch_bounds__(kWideThreads, 1) void varlen_attn_wide_kernel(AttnP
     }
     __syncthreads();
     const int n_parts = __builtin_amdgcn_readfirstlane(lds_plan[0]);
-    unsigned long long *stamps = reinterpret_cast<unsigned long long *>(p.ws_counters + 1024 + blockIdx.x * 64);
-    int n_stamp = 0;
-    if ((p.debug & 1024) && threadIdx.x == 0 && p.ws_counters) { stamps[1 + n_stamp++] = t_entry; stamps[30] = wall_clock64(); }
     for (int i = 0; i < n_parts; ++i) {
       attn_wide_part<DTYPE, D, MODE>(p, lds_ring, lds_tbl, lds_flag, lds_parts + i * kPlanInts, lds_par);
-      if ((p.debug & 1024) && threadIdx.x == 0 && p.ws_counters) {
-        stamps[1 + n_stamp++] = wall_clock64();
-        stamps[1 + n_stamp++] = ((unsigned long long)(lds_parts[i * kPlanInts + kPartTEnd] - lds_parts[i * kPlanInts + kPartTBegin]) << 32) |
-                                (unsigned)(lds_parts[i * kPlanInts + kPartNParts] * 16 + lds_parts[i * kPlanInts + kPartIndex]);
-        stamps[0] = n_stamp;
-      }
     }
     if (__builtin_amdgcn_readfirstlane(lds_plan[1]) == 0) break;
   }
