@@ -17,6 +17,8 @@ Additions with no single reference callable (documented at each function):
 """
 from __future__ import annotations
 
+import os
+
 import math
 from itertools import accumulate as _accumulate
 
@@ -548,6 +550,8 @@ def block_table_slots(
 
 
 _ATTN_WORKSPACES: dict = {}
+# same switch as the library reads: the 8-wave persistent kernel is taken only on request
+_ATTN_WIDE = os.environ.get("ACACHE_ATTN_WIDE", "")[:1] == "1"
 
 
 def attention_workspace(device) -> torch.Tensor:
@@ -587,7 +591,7 @@ def _varlen_attn(q, k_cache, v_cache, cu_q, cu_k, slots, scale, shared_prefix_le
     B = cu_q.numel() - 1
     rope_rows = 0 if cos is None else cos.shape[0]
     lib = _lib.load()
-    ws = attention_workspace(q.device)
+    ws = attention_workspace(q.device) if _ATTN_WIDE else None  # only the opt-in 8-wave kernel cuts units
     with torch.cuda.device(q.device):
         rc = lib.acache_varlen_attn(
             _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(cu_q), _ptr(cu_k), _ptr(slots),
