@@ -36,12 +36,12 @@ SIGNATURES = {
     "acache_affix_importance_workspace_bytes": (c_int64, [c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32]),
     "acache_affix_importance": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float,
-        c_int32, c_int64, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
+        c_int32, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
         c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p]),
     "acache_affix_importance_noalloc_max_bytes": (c_int64, []),
     "acache_affix_importance_noalloc": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_float,
-        c_int32, c_int64, c_int32, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
+        c_int32, c_int64, c_int32, c_int64, c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_int64,
         c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "acache_topk_anchors": (c_int32, [
         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_void_p]),

@@ -52,6 +52,13 @@ class Attention(nn.Module):
         scale = self.scale if self.scale is not None else self.head_dim ** -0.5
         if context.use_acache:
             q3 = q.reshape(-1, self.num_heads, self.head_dim) if q.dim() == 4 else q
+            if (self.shared_prefix_len > 0 and context.affix_shifts is not None and context.max_seqlen_k
+                    and self.relocation_rope_cos.shape[0] < context.max_seqlen_k):
+                # a shift is a position inside its request, so the longest request bounds every shift; the kernels
+                # only clamp out-of-table rows for memory safety and would return unrotated keys (the reference
+                # asserts the same bound after a device read-back, acache_attention.py:685)
+                raise ValueError(f"relocation RoPE table has {self.relocation_rope_cos.shape[0]} rows, "
+                                 f"the longest request needs {context.max_seqlen_k}")
             o = ops.acache_attention(
                 q3, k_cache, v_cache, context.cu_seqlens_q, context.cu_seqlens_k,
                 context.read_slot_mapping, scale, self.shared_prefix_len,

@@ -5,8 +5,11 @@
 //   w[r, h, a]       = softmax_a( q[r, h] . rot(K[a, kv(h)], shift_b) * scale )     a in [0, A)
 //   importance[b, a] += sum_{r in mask rows of b} sum_h w[r, h, a]
 //
-// Three launches (four with relocation: the cached keys of every request are first re-rotated once into the
-// workspace), no atomics, so the result does not depend on scheduling:
+// Relocation is applied on the query side: q . rot(k, +s) = rot(q, -s) . k, so with relocation a first launch
+// writes each request's [MASK] queries, rotated by minus the request's shift and packed in mask-row order, into
+// the workspace (a few hundred rows per request), and every launch after it reads the cached affix keys as they
+// lie in the cache: one copy of the keys, shared by all requests and resident in L2, instead of one re-rotated
+// copy per request.  Three more launches, no atomics, so the result does not depend on scheduling:
 //   1. importance_stats_kernel: one wave per (request, head, 64 mask rows) walks the affix keys and
 //      leaves the row maximum and the row sum of exp (log2 domain) in the workspace;
 //   2. importance_colsum_kernel: one wave per (request, head, 64 affix keys) keeps its keys in
@@ -35,8 +38,8 @@ struct ImportanceParams {
   const float *sin_tab;
   float2 *stats;
   float *partial;
-  char *k_rot;            // [B, A, H_kv, D] re-rotated affix keys (NULL: read the cache directly)
-  int64_t k_rot_bytes;    // per request
+  char *q_rot;            // [total_mask_rows, H, D] counter-rotated mask queries (NULL: read q through mask_rows)
+  int64_t total_q;        // rows of q; a mask row outside [0, total_q) is an absent query
   int64_t imp_stride;
   int64_t q_token_bytes, q_head_bytes;
   int64_t kv_slot_bytes, kv_head_bytes;
@@ -60,45 +63,46 @@ __device__ __forceinline__ void load_rows(vec16 (&f)[KS], const char *row_ptr, i
     f[ks] = row_ptr && 32 * ks + 8 * lg < head_dim ? load16(row_ptr + (32 * ks + 8 * lg) * 2) : vec16{{0, 0, 0, 0}};
 }
 
-// Re-rotate the cached affix keys once per request: k_rot[b, a, h, :] = rot(K[affix_slot0 + a, h, :], shift_b).
-// One row of D elements per LPR lanes, the rotate-half partner in the same lane; fp32 products and sum rounded
-// separately, one rounding to the cache type (the arithmetic of the relocation kernel).
+// Counter-rotate the [MASK] queries once per call: q_rot[m0_b + r, h, :] = rot(q[mask_rows[m0_b + r], h, :], -shift_b).
+// One row of D elements per D/16 lanes, the rotate-half partner in the same lane; fp32 products and sum rounded
+// separately, one rounding to the query type (the query-side arithmetic of the attention kernel).  A mask row
+// outside q is written as zeros (and counted as absent by the statistics kernel).
 template <int DTYPE>
 __global__ __launch_bounds__(256) void importance_rotate_kernel(ImportanceParams p) {
-#pragma clang fp contract(off)
-  using E = Elem<DTYPE>;
-  constexpr int VEC = E::kPerVec;
   const int D = p.D;
-  const int half_bytes = D * E::kBytes / 2;
+  const int half_bytes = D;  // D / 2 elements of 2 bytes
   const int lpr = half_bytes / 16;
   const int b = blockIdx.y;
+  const int m0 = p.cu_mask[b];
+  const int n_rows = p.cu_mask[b + 1] - m0;
   const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t row = g / lpr;
   const int lane = (int)(g - row * lpr);
-  if (row >= (int64_t)p.A * p.H_kv) return;
-  const int64_t a = row / p.H_kv;
-  const int head = (int)(row - a * p.H_kv);
-  int shift = p.shifts[b];
-  if (shift < 0 || shift >= p.rope_rows) shift = 0;
-  const char *src = p.k_cache + (p.affix_slot0 + a) * p.kv_slot_bytes + (int64_t)head * p.kv_head_bytes + lane * 16;
-  char *dst = p.k_rot + (int64_t)b * p.k_rot_bytes + row * (2 * half_bytes) + lane * 16;
-  vec16 lo = load16(src), hi = load16(src + half_bytes);
-  if (shift != 0) {
-    const float *cr = p.cos_tab + (int64_t)shift * D + lane * VEC;
-    const float *sr = p.sin_tab + (int64_t)shift * D + lane * VEC;
-    float x[VEC], y[VEC], xa[VEC], ya[VEC];
-    E::unpack(lo, x);
-    E::unpack(hi, y);
-#pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      xa[j] = x[j] * cr[j] + (-y[j]) * sr[j];
-      ya[j] = y[j] * cr[D / 2 + j] + x[j] * sr[D / 2 + j];
-    }
-    lo = E::pack(xa);
-    hi = E::pack(ya);
+  if (row >= (int64_t)n_rows * p.H) return;
+  const int r = (int)(row / p.H);
+  const int h = (int)(row - (int64_t)r * p.H);
+  char *dst = p.q_rot + (((int64_t)(m0 + r) * p.H + h) * D) * 2 + lane * 16;
+  const int64_t src_row = p.mask_rows[m0 + r];
+  vec16 lo = {{0, 0, 0, 0}}, hi = {{0, 0, 0, 0}};
+  if (src_row >= 0 && src_row < p.total_q) {
+    const char *src = p.q + src_row * p.q_token_bytes + (int64_t)h * p.q_head_bytes + lane * 16;
+    lo = load16(src);
+    hi = load16(src + half_bytes);
+    int shift = p.shifts[b];
+    if (shift < 0 || shift >= p.rope_rows) shift = 0;
+    if (shift != 0)
+      rotate_pair_half<DTYPE>(lo, hi, p.cos_tab + (int64_t)shift * D, p.sin_tab + (int64_t)shift * D, lane * 8, D / 2, -1.0f);
   }
   store16(dst, lo);
   store16(dst + half_bytes, hi);
+}
+
+// Row r of request b (first mask row m0), head h, as the scoring kernels read it: from the packed counter-rotated
+// copy when there is one, else from q through mask_rows; NULL (zeros) for a mask row outside q.
+__device__ __forceinline__ const char *mask_query_row(const ImportanceParams &p, int m0, int r, int h) {
+  if (p.q_rot) return p.q_rot + (((int64_t)(m0 + r) * p.H + h) * p.D) * 2;
+  const int64_t src_row = p.mask_rows[m0 + r];
+  return src_row >= 0 && src_row < p.total_q ? p.q + src_row * p.q_token_bytes + (int64_t)h * p.q_head_bytes : nullptr;
 }
 
 constexpr int kKeysPerStep = 64;  // keys a wave scores per loop step (four independent 16-key tiles in flight)
@@ -125,12 +129,10 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
     const int r = row0 + 16 * qt + li;
-    load_rows<KS>(qf[qt], r < n_rows ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
-                                     : nullptr, lg, D);
+    load_rows<KS>(qf[qt], r < n_rows ? mask_query_row(p, m0, r, h) : nullptr, lg, D);
   }
-  const int64_t slot_bytes = p.k_rot ? (int64_t)p.H_kv * D * 2 : p.kv_slot_bytes;
-  const char *k_base = p.k_rot ? p.k_rot + (int64_t)b * p.k_rot_bytes + (int64_t)kvh * D * 2
-                               : p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
+  const int64_t slot_bytes = p.kv_slot_bytes;
+  const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
   const float c = p.scale_log2e;
 
   float m_run[NQ], l_run[NQ];  // per query column (lane li); l is this lane group's share
@@ -176,7 +178,11 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
     l += __shfl_xor(l, 16);
     l += __shfl_xor(l, 32);
     const int r = row0 + 16 * qt + li;
-    if (lg == 0 && r < n_rows) p.stats[(int64_t)(m0 + r) * p.H + h] = make_float2(m_run[qt], l);
+    if (lg == 0 && r < n_rows) {
+      const int64_t src_row = p.mask_rows[m0 + r];
+      const bool present = src_row >= 0 && src_row < p.total_q;  // an absent query gets 1 / l = 0: it adds nothing
+      p.stats[(int64_t)(m0 + r) * p.H + h] = present ? make_float2(m_run[qt], l) : make_float2(0.0f, INFINITY);
+    }
   }
 }
 
@@ -196,9 +202,8 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
   if (h >= p.H) return;
   const float c = p.scale_log2e;
   const int kvh = h / (p.H / p.H_kv);
-  const int64_t slot_bytes = p.k_rot ? (int64_t)p.H_kv * D * 2 : p.kv_slot_bytes;
-  const char *k_base = p.k_rot ? p.k_rot + (int64_t)b * p.k_rot_bytes + (int64_t)kvh * D * 2
-                               : p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
+  const int64_t slot_bytes = p.kv_slot_bytes;
+  const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
 
   vec16 kf[4][KS];
 #pragma unroll
@@ -210,8 +215,7 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
   auto fetch = [&](int r0, vec16 (&qf)[KS], float2 &st) __attribute__((always_inline)) {
     const int r = r0 + li;
     const bool live = r < n_rows;
-    load_rows<KS>(qf, live ? p.q + (int64_t)p.mask_rows[m0 + r] * p.q_token_bytes + (int64_t)h * p.q_head_bytes
-                           : nullptr, lg, D);
+    load_rows<KS>(qf, live ? mask_query_row(p, m0, r, h) : nullptr, lg, D);
     st = live ? p.stats[(int64_t)(m0 + r) * p.H + h] : make_float2(0.0f, INFINITY);  // 1 / inf = 0: adds nothing
   };
   vec16 q_cur[KS], q_next[KS];
@@ -275,8 +279,8 @@ extern "C" int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_ro
                                                            int32_t H_kv, int32_t D, int32_t affix_len,
                                                            int32_t relocated) {
   if (total_mask_rows < 0 || B < 0 || H < 0 || H_kv < 0 || D < 0 || affix_len < 0) return 0;
-  if (relocated)  // one re-rotated copy of the affix keys per request (2-byte elements)
-    return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) + (int64_t)B * affix_len * H_kv * D * 2;
+  if (relocated)  // the counter-rotated copy of the mask queries (2-byte elements)
+    return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) + total_mask_rows * H * D * 2;
   return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len);
 }
 
@@ -284,7 +288,8 @@ extern "C" int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_ro
 static int importance_launch(
     float *importance, const void *q, const void *k_cache, const int32_t *mask_rows, const int32_t *cu_mask,
     const int32_t *affix_shifts, const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
-    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows, int32_t H,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_q, int64_t total_mask_rows, int32_t max_mask_rows,
+    int32_t H,
     int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t importance_stride, int64_t q_token_stride,
     int64_t q_head_stride, int64_t kv_slot_stride, int64_t kv_head_stride, void *workspace, int64_t workspace_bytes,
     void *stream) {
@@ -295,6 +300,8 @@ static int importance_launch(
   if (B < 0 || affix_len < 0 || total_mask_rows < 0 || max_mask_rows < 0 || H <= 0 || H_kv <= 0 || H % H_kv)
     return fail(ACACHE_E_SHAPE, "affix_importance: bad sizes (B %d, A %d, H %d, H_kv %d)", B, affix_len, H, H_kv);
   if (B == 0 || affix_len == 0 || total_mask_rows == 0 || max_mask_rows == 0) return 0;
+  if (total_q <= 0) return fail(ACACHE_E_SHAPE, "affix_importance: %lld mask rows but q has %lld rows",
+                                (long long)total_mask_rows, (long long)total_q);
   if (!importance || !q || !k_cache || !mask_rows || !cu_mask || !workspace)
     return fail(ACACHE_E_NULL, "affix_importance: NULL pointer");
   if (affix_shifts && (!rope_cos || !rope_sin || rope_rows <= 0))
@@ -316,8 +323,8 @@ static int importance_launch(
   p.mask_rows = mask_rows; p.cu_mask = cu_mask; p.shifts = affix_shifts;
   p.cos_tab = rope_cos; p.sin_tab = rope_sin; p.stats = (float2 *)workspace;
   p.partial = (float *)((char *)workspace + stats_bytes(total_mask_rows, H));
-  p.k_rot_bytes = (int64_t)affix_len * H_kv * D * 2;
-  p.k_rot = affix_shifts ? (char *)workspace + stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) : nullptr;
+  p.q_rot = affix_shifts ? (char *)workspace + stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) : nullptr;
+  p.total_q = total_q;
   p.imp_stride = importance_stride;
   p.q_token_bytes = q_token_stride * 2; p.q_head_bytes = q_head_stride * 2;
   p.kv_slot_bytes = kv_slot_stride * 2; p.kv_head_bytes = kv_head_stride * 2;
@@ -327,7 +334,7 @@ static int importance_launch(
   p.max_row_tiles = (max_mask_rows + 15) / 16;
   hipStream_t s = (hipStream_t)stream;
   const int lanes_per_row = D * 2 / 32;
-  const dim3 grid0((unsigned)(((int64_t)affix_len * H_kv * lanes_per_row + 255) / 256), (unsigned)B);
+  const dim3 grid0((unsigned)(((int64_t)max_mask_rows * H * lanes_per_row + 255) / 256), (unsigned)B);
   const int row_groups = (p.max_row_tiles + kRowTilesPerWave - 1) / kRowTilesPerWave;
   const dim3 grid1((unsigned)((int64_t)B * row_groups), (unsigned)((H + 3) / 4));
   const dim3 grid2((unsigned)((affix_len + kKeysPerStep - 1) / kKeysPerStep), (unsigned)((H + 3) / 4), (unsigned)B);
@@ -335,7 +342,7 @@ static int importance_launch(
   const int slabs = (D + 31) / 32;
 #define ACACHE_CASE(DT, SLABS)                                                                    \
   if (dtype == DT && slabs == SLABS) {                                                            \
-    if (p.k_rot) {                                                                                \
+    if (p.q_rot) {                                                                                \
       hipLaunchKernelGGL((importance_rotate_kernel<DT>), grid0, dim3(256), 0, s, p);              \
       const int rc0 = launch_status("importance_rotate_kernel");                                  \
       if (rc0) return rc0;                                                                        \
@@ -362,19 +369,20 @@ static int importance_launch(
 extern "C" int acache_affix_importance(
     float *importance, const void *q, const void *k_cache, const int32_t *mask_rows, const int32_t *cu_mask,
     const int32_t *affix_shifts, const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
-    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows, int32_t H,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_q, int64_t total_mask_rows, int32_t max_mask_rows,
+    int32_t H,
     int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t importance_stride, int64_t q_token_stride,
     int64_t q_head_stride, int64_t kv_slot_stride, int64_t kv_head_stride, void *workspace, int64_t workspace_bytes,
     void *stream) {
   return importance_launch(importance, q, k_cache, mask_rows, cu_mask, affix_shifts, rope_cos, rope_sin, rope_rows, scale,
-                           affix_len, affix_slot0, B, total_mask_rows, max_mask_rows, H, H_kv, D, dtype, num_slots,
+                           affix_len, affix_slot0, B, total_q, total_mask_rows, max_mask_rows, H, H_kv, D, dtype, num_slots,
                            importance_stride, q_token_stride, q_head_stride, kv_slot_stride, kv_head_stride, workspace,
                            workspace_bytes, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------
 // The same call for callers that cannot allocate device memory (code under HIP graph capture, serving
-// loops, harnesses that forbid hipMalloc): the row statistics, per-head partial sums and re-rotated keys
+// loops, harnesses that forbid hipMalloc): the row statistics, per-head partial sums and counter-rotated queries
 // live in a file-scope device array instead of a caller workspace.  Every GPU the library runs on holds
 // its own copy of the array at its own address until the process ends; the address is looked up once per
 // device and only that pointer is ever handed to kernels.  Nothing in the array has to start at zero:
@@ -411,7 +419,8 @@ extern "C" int64_t acache_affix_importance_noalloc_max_bytes(void) { return ACAC
 extern "C" int acache_affix_importance_noalloc(
     float *importance, const void *q, const void *k_cache, const int32_t *mask_rows, const int32_t *cu_mask,
     const int32_t *affix_shifts, const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
-    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows, int32_t H,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_q, int64_t total_mask_rows, int32_t max_mask_rows,
+    int32_t H,
     int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t importance_stride, int64_t q_token_stride,
     int64_t q_head_stride, int64_t kv_slot_stride, int64_t kv_head_stride, void *stream) {
   const int64_t need =
@@ -425,7 +434,7 @@ extern "C" int acache_affix_importance_noalloc(
   const int rc = scratch_of_current_device(&ws);
   if (rc) return rc;
   return importance_launch(importance, q, k_cache, mask_rows, cu_mask, affix_shifts, rope_cos, rope_sin, rope_rows, scale,
-                           affix_len, affix_slot0, B, total_mask_rows, max_mask_rows, H, H_kv, D, dtype, num_slots,
+                           affix_len, affix_slot0, B, total_q, total_mask_rows, max_mask_rows, H, H_kv, D, dtype, num_slots,
                            importance_stride, q_token_stride, q_head_stride, kv_slot_stride, kv_head_stride, ws,
                            ACACHE_IMPORTANCE_SCRATCH_BYTES, stream);
 }

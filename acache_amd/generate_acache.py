@@ -145,6 +145,16 @@ def _as_runner(model, *, mask_id, block_length, gen_length, anchor_ratio, select
         runner.config.block_length = block_length
         runner.config.gen_length = gen_length
         return runner
+    inner = getattr(model, "model", None)
+    engine_model = (inner is not None and hasattr(model, "config")
+                    and any(hasattr(m, "k_cache") and hasattr(m, "probe") for m in model.modules()))
+    if not engine_model:
+        # an HF checkpoint model attends over dense [B, H, L, D] caches inside its own forward; this entry point
+        # runs on the paged engine and cannot drive it
+        raise TypeError(
+            f"generate_ACache on this engine needs an acache_amd model (acache_amd.llada.LLaDAModelLM, "
+            f"acache_amd.dream.DreamModelLM) or a ready acache_amd.ModelRunner, got {type(model).__name__}: "
+            f"load the checkpoint's weights into the engine model first.")
     bs = 256
     blocks = 2 * (-(-affix_len // bs)) + -(-(total_len + affix_len) // bs) + 2
     cfg = Config(hf_config=model.config, mask_id=mask_id, recompute_batch_size=1, max_num_seqs=1,

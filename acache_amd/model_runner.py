@@ -18,13 +18,14 @@ loops.  What is re-designed:
   which the reference does for its Dream path only (model_runner.py:2101-2104);
 * the two generation loops share one implementation.
 
-Not carried over: the dKV-cache schedules (model_runner.py:1725-2030), the Dream
-decoder-layer variants and the CUDA-OOM shrink/retry of the KV cache
-(model_runner.py:592-638) — none is on the affix-KV reuse path measured here.
+Not carried over: the dKV-cache schedules (model_runner.py:1725-2030) and the Dream
+decoder-layer variants — neither is on the affix-KV reuse path measured here.
 """
 from __future__ import annotations
 
+import gc
 import math
+import sys
 import time
 
 import numpy as np
@@ -172,6 +173,12 @@ class ModelRunner:
         config.num_kvcache_blocks = int(num_blocks)
         assert config.num_kvcache_blocks >= 1, "Not enough GPU memory."
 
+        if self.kv_cache is not None:
+            # a resize: hand the old cache back before asking for the new one, or both are live at the peak
+            for module in self._attention_modules():
+                module.k_cache = module.v_cache = torch.empty(0, dtype=torch.bfloat16, device=self.device)
+            self.kv_cache = None
+            self._release_cached_device_memory()
         self.kv_cache = torch.empty(2, num_layers, config.num_kvcache_blocks, bs, num_kv_heads, head_dim,
                                     dtype=torch.bfloat16, device=self.device)
         self._reset_acache_state()
@@ -491,24 +498,100 @@ class ModelRunner:
                               affix_start=seq.prompt_affix_start, affix_end=seq.prompt_affix_end)
         return prefix
 
+    # KV-cache resize when admission runs out of device memory (model_runner.py:570-638, 862-955).  A resize
+    # rebuilds the cache and the block manager, so it is only allowed while no request is in flight.
+    def _blocks_for(self, prefix_len: int, private_blocks: int) -> int:
+        return max(-(-prefix_len // self.config.cache_block_size) + private_blocks, 1)
+
+    def _minimum_kv_cache_blocks_for_acache(self, seqs, prefix_len: int) -> int:
+        """Shared affix plus one whole request: below this nothing can be served."""
+        return self._blocks_for(prefix_len, max((s.num_cache_blocks for s in seqs), default=0))
+
+    def _selection_kv_cache_blocks(self, seqs, prefix_len: int) -> int:
+        """Shared affix plus the largest group of requests that one probe forward holds."""
+        step = int(getattr(self.config, "anchor_selection_batch_size", 1) or 0) or max(len(seqs), 1)
+        groups = (sum(s.num_cache_blocks for s in seqs[i:i + step]) for i in range(0, len(seqs), step))
+        return self._blocks_for(prefix_len, max(groups, default=0))
+
+    def _release_cached_device_memory(self):
+        gc.collect()
+        if self.device.type == "cuda":
+            torch.cuda.empty_cache()
+
+    def _shrink_kv_cache_for_acache(self, seqs, prefix_len: int, minimum_blocks: int | None = None) -> bool:
+        """Give up to four blocks back to the allocator; False when the cache is already at its floor."""
+        if self.kv_cache_block_bytes <= 0:
+            return False
+        floor = self._minimum_kv_cache_blocks_for_acache(seqs, prefix_len) if minimum_blocks is None else minimum_blocks
+        have = int(self.config.num_kvcache_blocks)
+        smaller = max(floor, have - 4)
+        if smaller >= have:
+            return False
+        print(f"[acache] anchor selection OOM, shrinking KV cache blocks from {have} to {smaller} and retrying.")
+        self.allocate_kv_cache(num_blocks=smaller)
+        return True
+
+    def _ensure_shared_prefix(self, prefix_token_ids, seqs, minimum_blocks: int | None = None):
+        """Affix precompute that answers an out-of-memory error by shrinking the KV cache and trying again."""
+        while True:
+            try:
+                self._precompute_shared_prefix(list(prefix_token_ids))
+                return
+            except torch.OutOfMemoryError as oom:
+                failure = torch.OutOfMemoryError(str(oom))   # a fresh object: the original pins the failed frames
+            self._release_cached_device_memory()
+            if not self._shrink_kv_cache_for_acache(seqs, len(prefix_token_ids), minimum_blocks):
+                raise failure
+
     def _select_anchor_positions_for_sequences(self, seqs, prefix_token_ids, allow_kv_cache_resize,
                                                minimum_blocks=None):
         # one request per probe forward by default, as the reference does (model_runner.py:873);
-        # Config.anchor_selection_batch_size widens the probe (0: all admitted requests in one forward)
+        # Config.anchor_selection_batch_size widens the probe (0: all admitted requests in one forward).
+        # Out of memory: first halve the probe group, then (if allowed) shrink the KV cache, redo the affix
+        # precompute that the new cache lost, and try the same group again.
         step = int(getattr(self.config, "anchor_selection_batch_size", 1) or 0) or len(seqs)
-        for i in range(0, len(seqs), step):
-            batch = seqs[i:i + step]
-            for seq, anchors in zip(batch, self._compute_anchor_positions_batch(batch)):
-                seq.set_anchor_positions(anchors)
+        done = 0
+        while done < len(seqs):
+            width = min(step, len(seqs) - done)
+            while True:
+                group = seqs[done:done + width]
+                try:
+                    for seq, anchors in zip(group, self._compute_anchor_positions_batch(group)):
+                        seq.set_anchor_positions(anchors)
+                    done += width
+                    break
+                except torch.OutOfMemoryError as oom:
+                    failure = torch.OutOfMemoryError(str(oom))
+                self._release_cached_device_memory()
+                if width > 1:
+                    width = max(width // 2, 1)
+                    continue
+                if not allow_kv_cache_resize or not self._shrink_kv_cache_for_acache(
+                        seqs, len(prefix_token_ids), minimum_blocks):
+                    raise failure
+                self._ensure_shared_prefix(prefix_token_ids, seqs, minimum_blocks)
 
     def _prepare_admitted_sequences_for_acache(self, seqs, prefix_token_ids, allow_kv_cache_resize):
         if not seqs:
             return
         if self.acache_ready and self.shared_prefix_token_ids != prefix_token_ids:
             raise ValueError("ACache prefix mode requires a consistent shared prefix across active requests.")
-        if not self.acache_ready:
-            self._precompute_shared_prefix(list(prefix_token_ids))
-        self._select_anchor_positions_for_sequences(seqs, prefix_token_ids, allow_kv_cache_resize)
+        target = int(self.config.num_kvcache_blocks)
+        floor = min(target, self._selection_kv_cache_blocks(seqs, len(prefix_token_ids)))
+        try:
+            if not self.acache_ready:
+                if allow_kv_cache_resize:
+                    self._ensure_shared_prefix(prefix_token_ids, seqs, floor)
+                else:
+                    self._precompute_shared_prefix(list(prefix_token_ids))
+            self._select_anchor_positions_for_sequences(seqs, prefix_token_ids, allow_kv_cache_resize, floor)
+        finally:
+            # selection is over (or failed): serving goes on with the cache size the caller configured
+            if allow_kv_cache_resize and self.config.num_kvcache_blocks != target:
+                failed = sys.exc_info()[0] is not None
+                self.allocate_kv_cache(num_blocks=target)
+                if not failed:
+                    self._ensure_shared_prefix(prefix_token_ids, seqs)
 
     def _finalize_sequence_layout(self, seq: Sequence):
         seq.finalize_slot_mapping()
@@ -773,7 +856,14 @@ class ModelRunner:
         refreshed = adjusted = False
         decoding_positions = None
         decode_graph = None
+        stalled = None   # device flag of the last refinement step: it left every [MASK] of its rows in place
         while batch:
+            if stalled is not None and bool(stalled):
+                # the committed tokens were all [MASK] again; the same forward would repeat for ever
+                raise RuntimeError(
+                    "Refinement step committed no token: the model predicts the mask token at every position "
+                    "still masked in the active blocks, so block-wise decoding cannot make progress.")
+            stalled = None
             has_mask = (working == mask_id).any(dim=1)
             done = ~has_mask
             if done.any():
@@ -845,6 +935,7 @@ class ModelRunner:
                                                        current_blocks, threshold)
                 r, c = torch.where(transfer)
                 working[active[r], c] = x0[transfer]
+                stalled = (working[active] == mask_id).sum() >= (current_blocks == mask_id).sum()
                 self._finish_timing(timing, "decode_update", start)
                 total_nfe += len(active)
 
@@ -911,9 +1002,14 @@ class ModelRunner:
         else:
             raise NotImplementedError(remasking)
         x0 = torch.where(mask_index, x0, x)
-        confidence = torch.where(mask_index, x0_p, torch.full_like(x0_p, -math.inf))
-        transfer = (confidence >= threshold) & mask_index
-        stuck = mask_index.any(dim=1) & ~transfer.any(dim=1)
+        # A position whose prediction is [MASK] itself cannot be committed: writing it changes nothing, and when it
+        # is the row's forced pick the same forward repeats for ever (the reference's rule, model_runner.py:2279-2314,
+        # never terminates there).  Such positions are left out of the pick; writing [MASK] over [MASK] is a no-op,
+        # so wherever the reference's loop terminates the committed tokens are the same.
+        committable = mask_index & (x0 != self.config.mask_id)
+        confidence = torch.where(committable, x0_p, torch.full_like(x0_p, -math.inf))
+        transfer = (confidence >= threshold) & committable
+        stuck = committable.any(dim=1) & ~transfer.any(dim=1)
         rows = torch.where(stuck)[0]
         transfer[rows, confidence.argmax(dim=1)[rows]] = True
         return x0, transfer

@@ -326,7 +326,8 @@ def affix_importance(
     """Add one layer's affix importance to ``importance`` (fp32 ``[B, >= affix_len]``).
 
     For each request the [MASK] queries ``q[mask_rows[cu_mask[b]:cu_mask[b+1]]]`` attend to the cached affix keys
-    ``k_cache`` slots ``affix_slot0 .. + affix_len`` (re-rotated by ``affix_shifts[b]``); the softmax runs over the
+    ``k_cache`` slots ``affix_slot0 .. + affix_len`` (relocated by ``affix_shifts[b]``: the queries are rotated by
+    the opposite angle, the keys are read as cached); the softmax runs over the
     affix keys only and its columns are summed over queries and heads (nano-vdllm/model_runner.py:730-773).
     ``workspace``: optional uint8 scratch of ``affix_importance_workspace_bytes`` bytes, allocated here if absent;
     the string ``"builtin"`` selects ``acache_affix_importance_noalloc``, which keeps its scratch in a fixed device
@@ -353,7 +354,7 @@ def affix_importance(
         _ptr(importance), _ptr(q), _ptr(kc), _ptr(rows), _ptr(cu), _ptr(shifts),
         _ptr(rope_cos) if relocate else None, _ptr(rope_sin) if relocate else None,
         rope_cos.shape[0] if relocate else 0, float(scale),
-        affix_len, affix_slot0, B, total, max_mask_rows, H, H_kv, D, _code(q), kc.shape[0],
+        affix_len, affix_slot0, B, Tq, total, max_mask_rows, H, H_kv, D, _code(q), kc.shape[0],
         importance.stride(0), q.stride(0), q.stride(1), kc.stride(0), kc.stride(1))
     if isinstance(workspace, str):
         if workspace != "builtin":
@@ -376,7 +377,7 @@ def affix_importance(
 def affix_importance_workspace_bytes(total_mask_rows: int, batch: int, num_heads: int, num_kv_heads: int,
                                      head_dim: int, affix_len: int, relocated: bool) -> int:
     """Bytes of scratch ``affix_importance`` needs: row statistics, per-head partial sums and, when
-    ``affix_shifts`` are given, one re-rotated copy of the affix keys per request."""
+    ``affix_shifts`` are given, the counter-rotated copy of the [MASK] queries."""
     return int(_lib.load().acache_affix_importance_workspace_bytes(
         total_mask_rows, batch, num_heads, num_kv_heads, head_dim, affix_len, int(relocated)))
 

@@ -348,11 +348,6 @@ def engine_bench(torch, device, args):
     with torch.device(device):
         model = LLaDAModelLM(cfg)
     model = model.to(torch.bfloat16).eval()
-    # A random output head predicts [MASK] itself once in ~126k tokens; such a position can never be committed
-    # and the decoding loop (the reference's as well) would spin on it.  Trained checkpoints do not do this, so
-    # the synthetic head gets a zero [MASK] row (logit 0, far below the maximum of 126k random logits).
-    with torch.no_grad():
-        model.model.transformer["ff_out"].weight[cfg.mask_token_id].zero_()
     rng = np.random.default_rng(0)
     vocab = np.array([t for t in range(cfg.vocab_size) if t != cfg.mask_token_id])
     affix = rng.choice(vocab, args.engine_affix).tolist()

@@ -172,21 +172,25 @@ int acache_rope_qk_scatter(
  * mask queries and the heads of one layer and ADDED to importance[b, :].
  *
  *   for b < B, r in mask_rows[cu_mask[b] .. cu_mask[b+1]), h < H:
- *     w[a] = softmax_a( q[r, h] . rot(k_cache[affix_slot0 + a, h / (H/H_kv)], affix_shifts[b]) * scale ), a < affix_len
+ *     w[a] = softmax_a( rot(q[r, h], -affix_shifts[b]) . k_cache[affix_slot0 + a, h / (H/H_kv)] * scale ), a < affix_len
  *     importance[b, a] += w[a]
- *   rot as in acache_relocate_rope_gather (rounded to `dtype`); fp32 scores and softmax.
+ *   rot(q, -s) = q*cos[s] - rot_half(q)*sin[s] in fp32, rounded once to `dtype` (the query-side
+ *   relocation of acache_varlen_attn); it equals q . rot(k, +s) before rounding.  fp32 scores and softmax.
  *
  * Replaces the per-request loop of the patched attention forward in
  * _compute_anchor_positions_batch (nano-vdllm/model_runner.py:730-773: rotary
  * re-application on the cached affix keys, matmul, softmax, two sums, add_), once
  * per layer; call it for every layer on the same importance buffer, then
  * acache_topk_anchors.  The reference evaluates matmul and softmax in the model
- * dtype; here they are fp32.  Deterministic: no atomics, fixed summation order.
+ * dtype and rounds the re-rotated keys to it; here scores and softmax are fp32 and the
+ * rotation (and its rounding) sits on the queries, so every request reads the one
+ * cached copy of the keys.  Deterministic: no atomics, fixed summation order.
  *
- * mask_rows are row indices into q ([Tq, H, D] with the given strides).  workspace:
+ * mask_rows are row indices into q ([total_q, H, D] with the given strides); an index outside
+ * [0, total_q) is an absent query and adds nothing.  workspace:
  * device scratch of at least acache_affix_importance_workspace_bytes(total_mask_rows, B, H,
  * H_kv, D, affix_len, relocated = affix_shifts != NULL) bytes (row statistics, per-head
- * partial sums and, with relocation, one re-rotated copy of the affix keys per request,
+ * partial sums and, with relocation, the counter-rotated copy of the mask queries,
  * passed between the launches), 16-byte aligned, owned by the caller.  max_mask_rows: an upper bound on
  * the mask rows of one request.  D: a multiple of 16 up to 256; dtype bf16 or f16.
  */
@@ -196,8 +200,8 @@ int acache_affix_importance(
     float *importance, const void *q, const void *k_cache,
     const int32_t *mask_rows, const int32_t *cu_mask, const int32_t *affix_shifts,
     const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
-    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows,
-    int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_q, int64_t total_mask_rows,
+    int32_t max_mask_rows, int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
     int64_t importance_stride, int64_t q_token_stride, int64_t q_head_stride,
     int64_t kv_slot_stride, int64_t kv_head_stride,
     void *workspace, int64_t workspace_bytes, void *stream);
@@ -218,14 +222,14 @@ int acache_affix_importance(
  * calls that overlap in time on the same GPU (different streams or threads) race; serialise
  * them.  The current device must be the one `stream` belongs to.
  */
-#define ACACHE_IMPORTANCE_SCRATCH_BYTES (32 << 20)
+#define ACACHE_IMPORTANCE_SCRATCH_BYTES (40 << 20)
 int64_t acache_affix_importance_noalloc_max_bytes(void);
 int acache_affix_importance_noalloc(
     float *importance, const void *q, const void *k_cache,
     const int32_t *mask_rows, const int32_t *cu_mask, const int32_t *affix_shifts,
     const float *rope_cos, const float *rope_sin, int32_t rope_rows, float scale,
-    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_mask_rows, int32_t max_mask_rows,
-    int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int32_t affix_len, int64_t affix_slot0, int32_t B, int64_t total_q, int64_t total_mask_rows,
+    int32_t max_mask_rows, int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
     int64_t importance_stride, int64_t q_token_stride, int64_t q_head_stride,
     int64_t kv_slot_stride, int64_t kv_head_stride, void *stream);
 

@@ -95,3 +95,20 @@ def test_coerce_bool_and_ceil():
     with pytest.raises(ValueError):
         _coerce_bool("maybe", False, "x")
     assert ceil_to_int(3.0) == 3 and ceil_to_int(3.0000001) == 4 and ceil_to_int(0.07 * 100) == math.ceil(0.07 * 100) == 8
+
+
+def test_foreign_models_are_rejected_with_a_type_error():
+    """The entry points keep the reference's signature but run on the paged engine: a model that is not built from
+    this package's attention modules (an HF checkpoint model, say) is refused before any device work."""
+    from acache_amd.generate_acache import generate_with_anchor_attention
+
+    class Foreign(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.model = torch.nn.Linear(4, 4)
+            self.config = object()
+
+    prompt = torch.arange(2, 10).unsqueeze(0)
+    with pytest.raises(TypeError, match="needs an acache_amd model"):
+        generate_with_anchor_attention(Foreign(), prompt, steps=4, gen_length=4, block_length=4, mask_id=MASK,
+                                       affix_start=0, affix_end=4)

@@ -54,6 +54,49 @@ def test_prepare_acache_tiny_model(device):
     assert runner.block_manager.used_block_ids == {0}
 
 
+def test_admission_out_of_memory_shrinks_the_cache_and_restores_it(device, capsys):
+    """An out-of-memory error in the anchor probe gives four KV blocks back, redoes the affix precompute in the
+    smaller cache, retries the same request, and ends with the configured cache size and a valid shared affix
+    (model_runner.py:592-638, 862-955).  The error is raised from the host; no allocation is actually refused."""
+    cfg, model = _model(device)
+
+    def requests():
+        return [Sequence([2, 3, 4, 5 + i], gen_length=4, cache_block_size=8, block_length=4, mask_id=63,
+                         prompt_affix_len=2) for i in range(2)]
+
+    def admit(fail_on, allow):
+        runner = ModelRunner(model, _serve(cfg, num_kvcache_blocks=12))
+        seqs = requests()
+        prefix = runner._prepare_acache(seqs)
+        real, sizes = runner._compute_anchor_positions_batch, []
+
+        def probe(batch):
+            sizes.append(int(runner.config.num_kvcache_blocks))
+            if len(sizes) == fail_on:
+                raise torch.OutOfMemoryError("forced by the test")
+            return real(batch)
+
+        runner._compute_anchor_positions_batch = probe
+        with torch.inference_mode():
+            runner._prepare_admitted_sequences_for_acache(seqs, prefix, allow_kv_cache_resize=allow)
+        return runner, seqs, sizes
+
+    plain, plain_seqs, sizes = admit(0, True)
+    assert sizes == [12, 12]
+    runner, seqs, sizes = admit(2, True)
+    assert sizes == [12, 12, 8]                      # second request: failed at 12 blocks, retried at 8
+    assert "shrinking KV cache blocks from 12 to 8" in capsys.readouterr().out
+    assert runner.config.num_kvcache_blocks == 12 and runner.kv_cache.shape[2] == 12
+    assert runner.acache_ready and runner.shared_prefix_token_ids == (2, 3)
+    assert runner.block_manager.used_block_ids == {0} and runner.block_manager.num_free_blocks == 11
+    assert [s.anchor_positions for s in seqs] == [s.anchor_positions for s in plain_seqs]
+    attn = runner._llada_blocks()[0].attn
+    assert attn.k_cache.data_ptr() == runner.kv_cache[0, 0].data_ptr()
+    assert torch.equal(runner._shared_affix_k(0), plain._shared_affix_k(0))
+    with pytest.raises(torch.OutOfMemoryError):
+        admit(1, False)
+
+
 def test_batched_anchor_selection_matches_single_sequence_selection(device):
     cfg, model = _model(device)
     serve = _serve(cfg, anchor_ratio=0.5)
@@ -212,8 +255,6 @@ def test_hip_graph_replay_of_refinement_steps_gives_the_same_tokens(device, use_
     transfer, scheduling, the next block's refresh) between replays; every run must commit exactly the tokens of the
     eager loop, and the graph must be re-captured when the attention metadata changes."""
     cfg, model = _model(device, seed=3)
-    with torch.no_grad():
-        model.model.transformer["ff_out"].weight[63].zero_()
     affix = list(range(20, 30))
 
     def make(i):

@@ -1,6 +1,7 @@
 """Affix-importance kernels against the oracle's fp32 restatement of nano-vdllm/model_runner.py:730-773.
-Both evaluate scores from the same bf16 inputs (re-rotated keys rounded to bf16) with fp32 accumulation and an
-fp32 softmax; they differ in summation order only: 2e-3 relative, 1e-4 absolute."""
+Both score bf16 operands with fp32 accumulation and an fp32 softmax.  The oracle, like the reference, re-rotates
+the cached keys and rounds them to bf16; the kernels rotate the queries by the opposite angle and round those
+(the same product before rounding), and they sum in another order: 2e-3 relative, 1e-4 absolute."""
 import pytest
 import torch
 
@@ -51,6 +52,20 @@ def test_no_relocation_f16_and_determinism(device):
     imp2 = torch.zeros_like(imp1)
     ops.affix_importance(imp2, q.to(device), kc.to(device), rows.to(device), cu.to(device), 130, 40, **args)
     assert torch.equal(imp1, imp2)                                        # no atomics: bit-identical reruns
+
+
+def test_mask_rows_outside_q_are_absent_queries(device):
+    """A stale or negative mask row must not be read: it counts as no query at all, with and without relocation."""
+    for shifts in (None, [9, 2]):
+        _, _, (q, kc, rows, cu, args) = _case(device, 8, 2, 128, A=90, mask_counts=[20, 6], shifts=shifts, seed=11)
+        clean = torch.zeros(2, 90, dtype=torch.float32, device=device)
+        ops.affix_importance(clean, q.to(device), kc.to(device), rows.to(device), cu.to(device), 90, 20, **args)
+        # splice three invalid indices into the first request's rows
+        bad = torch.cat([rows[:5], torch.tensor([-1, q.shape[0], 2 ** 30], dtype=torch.int32), rows[5:]])
+        cu_bad = torch.tensor([0, 23, 29], dtype=torch.int32)
+        got = torch.zeros_like(clean)
+        ops.affix_importance(got, q.to(device), kc.to(device), bad.to(device), cu_bad.to(device), 90, 23, **args)
+        assert torch.allclose(got, clean, rtol=1e-6, atol=1e-6)   # same rows, another tiling of them
 
 
 def test_argument_errors(device):

@@ -100,3 +100,100 @@ def test_collect_admissible_sequences_respects_free_blocks():
     assert got == seqs[:1] and nxt == 1            # 2 blocks each, 3 free -> one request
     got, nxt = runner._collect_admissible_sequences(seqs, 0, 0, 0)
     assert got == [] and nxt == 0
+
+
+class _StubForward:
+    """Stands in for the model in the generation loop: returns logits from a rule over the tokens it is shown, so
+    the loop's control flow runs on the CPU without any attention kernel."""
+
+    def __init__(self, rule, vocab=64):
+        self.rule, self.vocab, self.calls = rule, vocab, 0
+
+    def __call__(self, input_ids, position_ids=None, logits_keep_indices=None):
+        self.calls += 1
+        if logits_keep_indices is not None:      # cache refresh: one logit row per kept position
+            tokens = input_ids[logits_keep_indices]
+        else:                                    # block refinement: [requests, block_length]
+            tokens = input_ids
+        picks = self.rule(tokens)
+        logits = torch.zeros(*tokens.shape, self.vocab)
+        logits.scatter_(-1, picks.unsqueeze(-1), 4.0)
+        return SimpleNamespace(logits=logits)
+
+
+def _stub_requests(n=2):
+    return [Sequence([2 + i, 3, 4, 5], gen_length=8, cache_block_size=8, block_length=4, mask_id=63) for i in range(n)]
+
+
+def test_refinement_loop_raises_when_a_step_commits_nothing():
+    """A head that answers [MASK] everywhere can never fill a block: the loop must stop with an error instead of
+    repeating the same forward (the reference's loop, model_runner.py:1554-1723, has no such bound)."""
+    runner = _tiny_runner(num_kvcache_blocks=8, enable_acache=False, threshold=0.9)
+    runner.allocate_kv_cache(8)
+    runner.model = _StubForward(lambda tokens: torch.full_like(tokens, 63))
+    with pytest.raises(RuntimeError, match="committed no token"):
+        runner.generate_with_dual_cache(_stub_requests())
+    assert runner.model.calls <= 3   # one refresh forward, one refinement forward, no spin
+
+
+def test_forced_pick_skips_positions_that_predict_the_mask_token():
+    """Column 0 answers [MASK] until the rest of its block is filled, with the same confidence as every other
+    position; the forced one-token-per-step pick must take the other positions first and the run must finish."""
+    runner = _tiny_runner(num_kvcache_blocks=8, enable_acache=False, threshold=0.99)
+    runner.allocate_kv_cache(8)
+
+    def rule(tokens):
+        picks = torch.full_like(tokens, 7)
+        flat = tokens.reshape(-1, 4)
+        others_masked = (flat[:, 1:] == 63).any(dim=1)
+        picks.view(-1, 4)[others_masked, 0] = 63
+        return picks
+
+    runner.model = _StubForward(rule)
+    out, nfe = runner.generate_with_dual_cache(_stub_requests())
+    assert out == [[7] * 8, [7] * 8]
+    assert nfe == 2 * 2 * 4          # one token per request and step: 4 steps for each of 2 blocks of 2 requests
+
+
+def test_out_of_memory_at_admission_shrinks_retries_and_restores(capsys):
+    """Host logic of the resize path (model_runner.py:592-638, 862-955) with the two device steps stubbed: the
+    probe fails once with an out-of-memory error, the cache loses four blocks, the affix precompute is redone for
+    the new cache, the same request is retried, and the configured size is back afterwards."""
+    runner = _tiny_runner(num_kvcache_blocks=12)
+    runner.allocate_kv_cache(12)
+    seqs = [Sequence([2, 3, 4, 5 + i], gen_length=4, cache_block_size=8, block_length=4, mask_id=63,
+                     prompt_affix_len=2) for i in range(2)]
+    prefix = runner._prepare_acache(seqs)
+    log = []
+
+    def precompute(tokens):
+        log.append(("affix", int(runner.config.num_kvcache_blocks)))
+        runner.shared_prefix_len, runner.shared_prefix_blocks = len(tokens), 1
+        runner.shared_prefix_token_ids, runner.acache_ready = tuple(tokens), True
+
+    def probe(batch):
+        log.append(("probe", int(runner.config.num_kvcache_blocks)))
+        if sum(1 for what, _ in log if what == "probe") == 2:
+            raise torch.OutOfMemoryError("forced by the test")
+        return [[1] for _ in batch]
+
+    runner._precompute_shared_prefix = precompute
+    runner._compute_anchor_positions_batch = probe
+    runner._prepare_admitted_sequences_for_acache(seqs, prefix, allow_kv_cache_resize=True)
+    assert log == [("affix", 12), ("probe", 12), ("probe", 12), ("affix", 8), ("probe", 8), ("affix", 12)]
+    assert "from 12 to 8" in capsys.readouterr().out
+    assert runner.kv_cache.shape[2] == 12 and runner.block_manager.num_blocks == 12 and runner.acache_ready
+    assert [s.anchor_positions for s in seqs] == [[1], [1]]
+
+    # the floor: shared affix block + the one request a probe holds = 2 blocks; at the floor the error surfaces
+    runner.allocate_kv_cache(2)
+    log.clear()
+    runner._compute_anchor_positions_batch = lambda batch: (_ for _ in ()).throw(torch.OutOfMemoryError("always"))
+    with pytest.raises(torch.OutOfMemoryError):
+        runner._prepare_admitted_sequences_for_acache(seqs, prefix, allow_kv_cache_resize=True)
+    assert runner.kv_cache.shape[2] == 2
+    # without permission to resize nothing is shrunk
+    runner.allocate_kv_cache(12)
+    with pytest.raises(torch.OutOfMemoryError):
+        runner._prepare_admitted_sequences_for_acache(seqs, prefix, allow_kv_cache_resize=False)
+    assert runner.kv_cache.shape[2] == 12

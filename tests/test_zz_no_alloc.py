@@ -42,7 +42,7 @@ def _both(device, *case):
 
 
 def test_two_calls_share_the_builtin_scratch(device):
-    # LLaDA head geometry with relocation (the re-rotated keys live in the scratch too), then a smaller
+    # LLaDA head geometry with relocation (the counter-rotated queries live in the scratch too), then a smaller
     # request batch without relocation: stale contents of the first call must not leak into the second
     _both(device, 32, 32, 128, 300, [64, 40, 7], [5, 0, 130], 1)
     _both(device, 8, 2, 128, 70, [9, 0, 3], None, 2)
@@ -53,14 +53,14 @@ def test_two_calls_share_the_builtin_scratch(device):
 def test_oversized_call_is_rejected_before_any_launch(device):
     lib = _lib.load()
     limit = lib.acache_affix_importance_noalloc_max_bytes()
-    assert limit == 32 << 20
+    assert limit == 40 << 20
     q, kc, rows, cu, A, max_rows, kw = _inputs(device, 4, 4, 128, 50, [4], None, 4)
     imp = torch.zeros(1, A, dtype=torch.float32, device=device)
     # claim more mask rows than the array can keep statistics for: rejected from the sizes alone
     too_many = limit // (4 * 8) + 1
     rc = lib.acache_affix_importance_noalloc(
         imp.data_ptr(), q.data_ptr(), kc.data_ptr(), rows.data_ptr(), cu.data_ptr(), None, None, None, 0,
-        float(128 ** -0.5), A, 0, 1, too_many, 4, 4, 4, 128, 0, kc.shape[0], imp.stride(0), q.stride(0), q.stride(1),
+        float(128 ** -0.5), A, 0, 1, q.shape[0], too_many, 4, 4, 4, 128, 0, kc.shape[0], imp.stride(0), q.stride(0), q.stride(1),
         kc.stride(0), kc.stride(1), None)
     assert rc == -3 and b"built-in buffer" in lib.acache_last_error()
     torch.cuda.synchronize(device)
