@@ -5,22 +5,24 @@
 //   w[r, h, a]       = softmax_a( q[r, h] . rot(K[a, kv(h)], shift_b) * scale )     a in [0, A)
 //   importance[b, a] += sum_{r in mask rows of b} sum_h w[r, h, a]
 //
-// Relocation is applied on the query side: q . rot(k, +s) = rot(q, -s) . k, so with relocation a first launch
-// writes each request's [MASK] queries, rotated by minus the request's shift and packed in mask-row order, into
-// the workspace (a few hundred rows per request), and every launch after it reads the cached affix keys as they
-// lie in the cache: one copy of the keys, shared by all requests and resident in L2, instead of one re-rotated
-// copy per request.  Three more launches, no atomics, so the result does not depend on scheduling:
+// Relocation is applied on the query side: q . rot(k, +s) = rot(q, -s) . k.  A first launch writes each request's
+// [MASK] queries, packed in mask-row order and (with relocation) rotated by minus the request's shift, into the
+// workspace (a few hundred rows per request); every launch after it reads that copy without an index in between
+// and the cached affix keys as they lie in the cache: one copy of the keys, shared by all requests and resident
+// in L2, instead of one re-rotated copy per request.  Three more launches, no atomics, so the result does not
+// depend on scheduling:
 //   1. importance_stats_kernel: one wave per (request, head, 64 mask rows) walks the affix keys and
-//      leaves the row maximum and the row sum of exp (log2 domain) in the workspace;
+//      leaves log2 of the row's sum of 2^(score * c) in the workspace;
 //   2. importance_colsum_kernel: one wave per (request, head, 64 affix keys) keeps its keys in
 //      registers, walks the request's mask rows, recomputes the scores, normalises them with the
-//      stored row statistics and sums the columns; it is the only writer of its 64 entries of the
+//      stored row statistic (one subtraction in the exponent) and sums the columns; it is the only writer of its 64 entries of the
 //      per-head partial sums in the workspace;
 //   3. importance_reduce_kernel adds the per-head partial sums, in head order, to importance[b, :].
 // Scores come from the matrix core (S^T = K Q^T, keys as rows, one query column per lane).  K and Q
 // fragments are loaded straight from global memory in operand layout (16 bytes per lane); nothing goes
 // through LDS and there is no barrier.
 #include <mutex>
+#include <type_traits>
 
 #include "common.h"
 #include "mma.h"
@@ -36,9 +38,9 @@ struct ImportanceParams {
   const int32_t *shifts;
   const float *cos_tab;
   const float *sin_tab;
-  float2 *stats;
+  float *stats;            // per (mask row, head): log2 of the row's sum of 2^(score * c)
   float *partial;
-  char *q_rot;            // [total_mask_rows, H, D] counter-rotated mask queries (NULL: read q through mask_rows)
+  char *q_rot;            // [total_mask_rows, H, D] mask queries packed in mask-row order, counter-rotated
   int64_t total_q;        // rows of q; a mask row outside [0, total_q) is an absent query
   int64_t imp_stride;
   int64_t q_token_bytes, q_head_bytes;
@@ -54,13 +56,21 @@ struct ImportanceParams {
   int32_t D;  // head_dim
 };
 
-// Operand fragments of 16 rows x head_dim, KS slabs of 32 elements: lane (li, lg) takes row `row_ptr`
-// (NULL: zeros), elements 32*ks + 8*lg .. + 8; chunks at or past head_dim (a multiple of 16) read as zeros.
-template <int KS>
-__device__ __forceinline__ void load_rows(vec16 (&f)[KS], const char *row_ptr, int lg, int head_dim) {
+// Operand fragments of 16 rows x D, KS = ceil(D / 32) slabs of 32 elements: lane (li, lg) takes elements
+// 32*ks + 8*lg .. + 8 of row `row_ptr` (always a readable row: callers clamp indices instead of branching, so
+// the loads of a tile issue back to back); chunks at or past D (a multiple of 16) read as zeros.
+template <int D>
+__device__ __forceinline__ void load_rows(vec16 (&f)[(D + 31) / 32], const char *row_ptr, int lg) {
+  constexpr int KS = (D + 31) / 32;
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks)
-    f[ks] = row_ptr && 32 * ks + 8 * lg < head_dim ? load16(row_ptr + (32 * ks + 8 * lg) * 2) : vec16{{0, 0, 0, 0}};
+  for (int ks = 0; ks < KS; ++ks) {
+    if (32 * ks + 32 <= D) {
+      f[ks] = load16(row_ptr + (32 * ks + 8 * lg) * 2);
+    } else {  // the half-filled last slab of D = 16 (mod 32): lane groups 2 and 3 hold zeros
+      const vec16 v = load16(row_ptr + (32 * ks + 8 * (lg & 1)) * 2);
+      f[ks] = lg < 2 ? v : vec16{{0, 0, 0, 0}};
+    }
+  }
 }
 
 // Counter-rotate the [MASK] queries once per call: q_rot[m0_b + r, h, :] = rot(q[mask_rows[m0_b + r], h, :], -shift_b).
@@ -88,7 +98,7 @@ __global__ __launch_bounds__(256) void importance_rotate_kernel(ImportanceParams
     const char *src = p.q + src_row * p.q_token_bytes + (int64_t)h * p.q_head_bytes + lane * 16;
     lo = load16(src);
     hi = load16(src + half_bytes);
-    int shift = p.shifts[b];
+    int shift = p.shifts ? p.shifts[b] : 0;
     if (shift < 0 || shift >= p.rope_rows) shift = 0;
     if (shift != 0)
       rotate_pair_half<DTYPE>(lo, hi, p.cos_tab + (int64_t)shift * D, p.sin_tab + (int64_t)shift * D, lane * 8, D / 2, -1.0f);
@@ -97,22 +107,35 @@ __global__ __launch_bounds__(256) void importance_rotate_kernel(ImportanceParams
   store16(dst + half_bytes, hi);
 }
 
-// Row r of request b (first mask row m0), head h, as the scoring kernels read it: from the packed counter-rotated
-// copy when there is one, else from q through mask_rows; NULL (zeros) for a mask row outside q.
-__device__ __forceinline__ const char *mask_query_row(const ImportanceParams &p, int m0, int r, int h) {
-  if (p.q_rot) return p.q_rot + (((int64_t)(m0 + r) * p.H + h) * p.D) * 2;
-  const int64_t src_row = p.mask_rows[m0 + r];
-  return src_row >= 0 && src_row < p.total_q ? p.q + src_row * p.q_token_bytes + (int64_t)h * p.q_head_bytes : nullptr;
+// Row r of request b (first mask row m0), head h, in the packed copy the first launch wrote.  Always a readable
+// address: r is clamped to the request's rows (callers discard what a clamped row contributes).  The copy is
+// smaller than 4 GiB (checked at launch), so the offset is 32-bit arithmetic.
+__device__ __forceinline__ const char *mask_query_row(const ImportanceParams &p, int m0, int n_rows, int r, int h) {
+  r = r < n_rows ? r : n_rows - 1;
+  return p.q_rot + ((uint32_t)(m0 + r) * (uint32_t)p.H + (uint32_t)h) * (uint32_t)(p.D * 2);
 }
 
-constexpr int kKeysPerStep = 64;  // keys a wave scores per loop step (four independent 16-key tiles in flight)
+// Sum over the 16 lanes of a row (lanes sharing lane >> 4), left in every lane of the row: four rotate-and-add
+// steps in the vector ALU's lane-permute path (no trip through LDS).
+__device__ __forceinline__ float row_sum16(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+  return v;
+}
+
+constexpr int kKeysPerStep = 64;  // keys a colsum wave owns (four independent 16-key tiles in flight)
+constexpr int kStatKeys = 32;     // keys a stats wave scores per loop step (two 16-key tiles x two row tiles in flight)
 
 constexpr int kRowTilesPerWave = 4;  // 16-row tiles of mask queries a stats wave owns (keys are loaded once for all)
 
-template <int DTYPE, int KS>
+// One wave per (request, head, 64 mask rows): the rows stay in registers, the affix keys stream by, and the wave
+// leaves log2(sum_a 2^(s[r, a] * c)) per row (running maximum + log2 of the running sum) in the workspace.
+template <int DTYPE, int D>
 __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams p) {
   constexpr int NQ = kRowTilesPerWave;
-  const int D = p.D;  // KS = ceil(D / 32) slabs; the last one may be half empty
+  constexpr int KS = (D + 31) / 32;
   using M = Mma<DTYPE>;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
@@ -127,50 +150,73 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
 
   vec16 qf[NQ][KS];
 #pragma unroll
-  for (int qt = 0; qt < NQ; ++qt) {
-    const int r = row0 + 16 * qt + li;
-    load_rows<KS>(qf[qt], r < n_rows ? mask_query_row(p, m0, r, h) : nullptr, lg, D);
-  }
-  const int64_t slot_bytes = p.kv_slot_bytes;
+  for (int qt = 0; qt < NQ; ++qt) load_rows<D>(qf[qt], mask_query_row(p, m0, n_rows, row0 + 16 * qt + li, h), lg);
   const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
   const float c = p.scale_log2e;
 
   float m_run[NQ], l_run[NQ];  // per query column (lane li); l is this lane group's share
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) { m_run[qt] = -INFINITY; l_run[qt] = 0.0f; }
-  for (int a0 = 0; a0 < p.A; a0 += kKeysPerStep) {
-    vec16 kf[4][KS];  // 64 keys: rows a0 + 16*nt + li
+  constexpr int NT = kStatKeys / 16;
+  // keys a0 + 16*nt + li of one step, clamped to the affix (a clamped key is masked out below)
+  auto fetch = [&](int a0, vec16 (&kf)[NT][KS]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
+    for (int nt = 0; nt < NT; ++nt) {
       const int a = a0 + 16 * nt + li;
-      load_rows<KS>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, D);
+      load_rows<D>(kf[nt], k_base + (int64_t)(a < p.A ? a : p.A - 1) * p.kv_slot_bytes, lg);
     }
+  };
+  // one step on the keys in `kf`, with the next step's keys requested first (always: past the end the clamped
+  // addresses are re-read and the result ignored, which keeps the loop free of a branch the loads would wait at)
+  auto step = [&](int a0, vec16 (&kf)[NT][KS], vec16 (&kf_next)[NT][KS]) __attribute__((always_inline)) {
+    fetch(a0 + kStatKeys, kf_next);
+    const bool tail = a0 + kStatKeys > p.A;  // wave-uniform: only the last step holds keys past the affix
 #pragma unroll
-    for (int qt = 0; qt < NQ; ++qt) {
-      f32x4 s[4];
-      float mx = -INFINITY;
+    for (int qp = 0; qp < NQ; qp += 2) {  // two row tiles at a time: four independent accumulator chains
+      f32x4 sc[2][NT];
 #pragma unroll
-      for (int nt = 0; nt < 4; ++nt) {
-        s[nt] = f32x4{0, 0, 0, 0};
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) s[nt] = M::run(kf[nt][ks], qf[qt][ks], s[nt]);
+        for (int nt = 0; nt < NT; ++nt) sc[u][nt] = f32x4{0, 0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (a0 + 16 * nt + 4 * lg + i >= p.A) s[nt][i] = -INFINITY;
-          mx = fmaxf(mx, s[nt][i]);
+      for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) sc[u][nt] = M::run(kf[nt][ks], qf[qp + u][ks], sc[u][nt]);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int qt = qp + u;
+        if (tail) {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (a0 + 16 * nt + 4 * lg + i >= p.A) sc[u][nt][i] = -INFINITY;
         }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sc[u][nt][i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run[qt], mx * c);  // finite: every step holds at least one existing key
+        float add = 0.0f;
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(sc[u][nt][i] * c - m_new);
+        l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + add;
+        m_run[qt] = m_new;
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run[qt], mx * c);  // finite: every step holds at least one existing key
-      float add = 0.0f;
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(s[nt][i] * c - m_new);
-      l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + add;
-      m_run[qt] = m_new;
     }
+  };
+  vec16 kf_a[NT][KS], kf_b[NT][KS];
+  fetch(0, kf_a);
+  for (int a0 = 0; a0 < p.A; a0 += 2 * kStatKeys) {
+    step(a0, kf_a, kf_b);
+    if (a0 + kStatKeys < p.A) step(a0 + kStatKeys, kf_b, kf_a);
   }
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
@@ -180,18 +226,21 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
     const int r = row0 + 16 * qt + li;
     if (lg == 0 && r < n_rows) {
       const int64_t src_row = p.mask_rows[m0 + r];
-      const bool present = src_row >= 0 && src_row < p.total_q;  // an absent query gets 1 / l = 0: it adds nothing
-      p.stats[(int64_t)(m0 + r) * p.H + h] = present ? make_float2(m_run[qt], l) : make_float2(0.0f, INFINITY);
+      const bool present = src_row >= 0 && src_row < p.total_q;  // an absent query gets 2^-inf = 0: it adds nothing
+      p.stats[(int64_t)(m0 + r) * p.H + h] = present ? m_run[qt] + __builtin_amdgcn_logf(l) : INFINITY;
     }
   }
 }
 
-// One wave per (request, head, 64 affix keys): the keys stay in registers, the request's mask rows stream by.
-// The wave is the only writer of partial[b, h, a0 .. a0 + 64).
-template <int DTYPE, int KS>
+constexpr int kColRowTiles = 2;  // 16-row tiles of mask queries a colsum wave scores per loop step
+
+// One wave per (request, head, 64 affix keys): the keys stay in registers, the request's mask rows stream by
+// 32 at a time (the next 32 already on their way).  The wave is the only writer of partial[b, h, a0 .. a0 + 64).
+template <int DTYPE, int D>
 __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams p) {
+  constexpr int KS = (D + 31) / 32;
+  constexpr int NR = kColRowTiles;
   using M = Mma<DTYPE>;
-  const int D = p.D;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int li = lane & 15, lg = lane >> 4;
   const int b = blockIdx.z;
@@ -202,39 +251,52 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
   if (h >= p.H) return;
   const float c = p.scale_log2e;
   const int kvh = h / (p.H / p.H_kv);
-  const int64_t slot_bytes = p.kv_slot_bytes;
   const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
 
-  vec16 kf[4][KS];
+  vec16 kf[4][KS];  // keys past the affix repeat the last one; their columns are not stored
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
     const int a = a0 + 16 * nt + li;
-    load_rows<KS>(kf[nt], a < p.A ? k_base + (int64_t)a * slot_bytes : nullptr, lg, D);
+    load_rows<D>(kf[nt], k_base + (int64_t)(a < p.A ? a : p.A - 1) * p.kv_slot_bytes, lg);
   }
   float col[4][4] = {};
-  auto fetch = [&](int r0, vec16 (&qf)[KS], float2 &st) __attribute__((always_inline)) {
-    const int r = r0 + li;
-    const bool live = r < n_rows;
-    load_rows<KS>(qf, live ? mask_query_row(p, m0, r, h) : nullptr, lg, D);
-    st = live ? p.stats[(int64_t)(m0 + r) * p.H + h] : make_float2(0.0f, INFINITY);  // 1 / inf = 0: adds nothing
-  };
-  vec16 q_cur[KS], q_next[KS];
-  float2 st_cur, st_next;
-  if (n_rows > 0) fetch(0, q_cur, st_cur);
-  for (int r0 = 0; r0 < n_rows; r0 += 16) {
-    if (r0 + 16 < n_rows) fetch(r0 + 16, q_next, st_next);  // next row tile on its way while this one is scored
-    const float inv_l = 1.0f / st_cur.y;
+  auto fetch = [&](int r0, vec16 (&qf)[NR][KS], float (&st)[NR]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      f32x4 s = {0, 0, 0, 0};
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) s = M::run(kf[nt][ks], q_cur[ks], s);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(s[i] * c - st_cur.x) * inv_l;
+    for (int t = 0; t < NR; ++t) {
+      const int r = r0 + 16 * t + li;
+      load_rows<D>(qf[t], mask_query_row(p, m0, n_rows, r, h), lg);
+      st[t] = p.stats[(int64_t)(m0 + (r < n_rows ? r : n_rows - 1)) * p.H + h];
     }
+  };
+  // one step on the 32 rows in `qf`, with the next 32 requested first (always: past the end the clamped rows are
+  // re-read and ignored, which keeps the loop free of a branch the loads would wait at)
+  auto step = [&](int r0, vec16 (&qf)[NR][KS], float (&st)[NR], vec16 (&qf_next)[NR][KS], float (&st_next)[NR])
+      __attribute__((always_inline)) {
+    fetch(r0 + 16 * NR, qf_next, st_next);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) q_cur[ks] = q_next[ks];
-    st_cur = st_next;
+    for (int t = 0; t < NR; ++t) {
+      // a row past the request's end was read from a clamped address: 2^-inf = 0 keeps it out of the sums (the
+      // test sits here, not at the load, so that the prefetch is not waited for the moment it is issued)
+      const float ref = r0 + 16 * t + li < n_rows ? st[t] : INFINITY;
+      f32x4 sc[4];
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) sc[nt] = f32x4{0, 0, 0, 0};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)  // four independent accumulator chains between two steps of one chain
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) sc[nt] = M::run(kf[nt][ks], qf[t][ks], sc[nt]);
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(sc[nt][i] * c - ref);
+    }
+  };
+  vec16 q_a[NR][KS], q_b[NR][KS];
+  float st_a[NR], st_b[NR];
+  if (n_rows > 0) fetch(0, q_a, st_a);
+  for (int r0 = 0; r0 < n_rows; r0 += 32 * NR) {
+    step(r0, q_a, st_a, q_b, st_b);
+    if (r0 + 16 * NR < n_rows) step(r0 + 16 * NR, q_b, st_b, q_a, st_a);
   }
   // sum over the 16 query columns (lanes li) of every key row
   float *dst = p.partial + ((int64_t)b * p.H + h) * p.A;
@@ -242,25 +304,31 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
   for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float v = col[nt][i];
-      v += __shfl_xor(v, 1);
-      v += __shfl_xor(v, 2);
-      v += __shfl_xor(v, 4);
-      v += __shfl_xor(v, 8);
+      const float v = row_sum16(col[nt][i]);
       const int a = a0 + 16 * nt + 4 * lg + i;
       if (li == 0 && a < p.A) dst[a] = v;
     }
 }
 
-// importance[b, a] += sum over heads, in head order, of partial[b, h, a].
+// importance[b, a] += sum over heads of partial[b, h, a], in a fixed order: four lanes take every fourth head
+// each (their loads all in flight together), then the four shares are added in lane order.
 __global__ __launch_bounds__(256) void importance_reduce_kernel(ImportanceParams p) {
-  const int a = blockIdx.x * 256 + threadIdx.x;
+  __shared__ float share[4][64];
+  const int a = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int part = threadIdx.x >> 6;
   const int b = blockIdx.y;
-  if (a >= p.A) return;
-  const float *src = p.partial + (int64_t)b * p.H * p.A + a;
   float acc = 0.0f;
-  for (int h = 0; h < p.H; ++h) acc += src[(int64_t)h * p.A];
-  p.importance[(int64_t)b * p.imp_stride + a] += acc;
+  if (a < p.A) {
+    const float *src = p.partial + (int64_t)b * p.H * p.A + a;
+#pragma unroll 8
+    for (int h = part; h < p.H; h += 4) acc += src[(int64_t)h * p.A];
+  }
+  share[part][threadIdx.x & 63] = acc;
+  __syncthreads();
+  if (part == 0 && a < p.A) {
+    const int j = threadIdx.x;
+    p.importance[(int64_t)b * p.imp_stride + a] += ((share[0][j] + share[1][j]) + share[2][j]) + share[3][j];
+  }
 }
 
 }  // namespace acache
@@ -268,7 +336,7 @@ __global__ __launch_bounds__(256) void importance_reduce_kernel(ImportanceParams
 using namespace acache;
 
 static int64_t stats_bytes(int64_t total_mask_rows, int32_t H) {
-  return (total_mask_rows * H * (int64_t)sizeof(float2) + 15) / 16 * 16;
+  return (total_mask_rows * H * (int64_t)sizeof(float) + 15) / 16 * 16;
 }
 
 static int64_t partial_bytes(int32_t B, int32_t H, int32_t affix_len) {
@@ -279,9 +347,9 @@ extern "C" int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_ro
                                                            int32_t H_kv, int32_t D, int32_t affix_len,
                                                            int32_t relocated) {
   if (total_mask_rows < 0 || B < 0 || H < 0 || H_kv < 0 || D < 0 || affix_len < 0) return 0;
-  if (relocated)  // the counter-rotated copy of the mask queries (2-byte elements)
-    return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) + total_mask_rows * H * D * 2;
-  return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len);
+  (void)H_kv;
+  (void)relocated;  // the packed copy of the mask queries (2-byte elements) is made with and without relocation
+  return stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) + total_mask_rows * H * D * 2;
 }
 
 // Argument checks and the launches; `workspace` is caller memory or this library's file-scope scratch.
@@ -311,6 +379,9 @@ static int importance_launch(
     return fail(ACACHE_E_RANGE, "affix_importance: affix slots [%lld, %lld) outside %lld slots", (long long)affix_slot0,
                 (long long)(affix_slot0 + affix_len), (long long)num_slots);
   if (importance_stride < affix_len) return fail(ACACHE_E_SHAPE, "affix_importance: importance stride < affix_len");
+  if (total_mask_rows * H * D * 2 >= ((int64_t)1 << 32))
+    return fail(ACACHE_E_SHAPE, "affix_importance: %lld mask rows x %d heads x %d: the packed query copy must stay under 4 GiB",
+                (long long)total_mask_rows, H, D);
   if (workspace_bytes < acache_affix_importance_workspace_bytes(total_mask_rows, B, H, H_kv, D, affix_len, affix_shifts != nullptr))
     return fail(ACACHE_E_SHAPE, "affix_importance: workspace of %lld bytes, %lld needed", (long long)workspace_bytes,
                 (long long)acache_affix_importance_workspace_bytes(total_mask_rows, B, H, H_kv, D, affix_len, affix_shifts != nullptr));
@@ -321,9 +392,9 @@ static int importance_launch(
   ImportanceParams p;
   p.importance = importance; p.q = (const char *)q; p.k_cache = (const char *)k_cache;
   p.mask_rows = mask_rows; p.cu_mask = cu_mask; p.shifts = affix_shifts;
-  p.cos_tab = rope_cos; p.sin_tab = rope_sin; p.stats = (float2 *)workspace;
+  p.cos_tab = rope_cos; p.sin_tab = rope_sin; p.stats = (float *)workspace;
   p.partial = (float *)((char *)workspace + stats_bytes(total_mask_rows, H));
-  p.q_rot = affix_shifts ? (char *)workspace + stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len) : nullptr;
+  p.q_rot = (char *)workspace + stats_bytes(total_mask_rows, H) + partial_bytes(B, H, affix_len);
   p.total_q = total_q;
   p.imp_stride = importance_stride;
   p.q_token_bytes = q_token_stride * 2; p.q_head_bytes = q_head_stride * 2;
@@ -338,30 +409,29 @@ static int importance_launch(
   const int row_groups = (p.max_row_tiles + kRowTilesPerWave - 1) / kRowTilesPerWave;
   const dim3 grid1((unsigned)((int64_t)B * row_groups), (unsigned)((H + 3) / 4));
   const dim3 grid2((unsigned)((affix_len + kKeysPerStep - 1) / kKeysPerStep), (unsigned)((H + 3) / 4), (unsigned)B);
-  const dim3 grid3((unsigned)((affix_len + 255) / 256), (unsigned)B);
-  const int slabs = (D + 31) / 32;
-#define ACACHE_CASE(DT, SLABS)                                                                    \
-  if (dtype == DT && slabs == SLABS) {                                                            \
-    if (p.q_rot) {                                                                                \
-      hipLaunchKernelGGL((importance_rotate_kernel<DT>), grid0, dim3(256), 0, s, p);              \
-      const int rc0 = launch_status("importance_rotate_kernel");                                  \
-      if (rc0) return rc0;                                                                        \
-    }                                                                                             \
-    hipLaunchKernelGGL((importance_stats_kernel<DT, SLABS>), grid1, dim3(256), 0, s, p);          \
+  const dim3 grid3((unsigned)((affix_len + 63) / 64), (unsigned)B);
+#define ACACHE_CASE(DT, HD)                                                                       \
+  if (dtype == DT && D == HD) {                                                                   \
+    hipLaunchKernelGGL((importance_rotate_kernel<DT>), grid0, dim3(256), 0, s, p);                \
+    const int rc0 = launch_status("importance_rotate_kernel");                                    \
+    if (rc0) return rc0;                                                                          \
+    hipLaunchKernelGGL((importance_stats_kernel<DT, HD>), grid1, dim3(256), 0, s, p);             \
     const int rc = launch_status("importance_stats_kernel");                                      \
     if (rc) return rc;                                                                            \
-    hipLaunchKernelGGL((importance_colsum_kernel<DT, SLABS>), grid2, dim3(256), 0, s, p);         \
+    hipLaunchKernelGGL((importance_colsum_kernel<DT, HD>), grid2, dim3(256), 0, s, p);            \
     const int rc2 = launch_status("importance_colsum_kernel");                                    \
     if (rc2) return rc2;                                                                          \
     hipLaunchKernelGGL(importance_reduce_kernel, grid3, dim3(256), 0, s, p);                      \
     return launch_status("importance_reduce_kernel");                                             \
   }
-#define ACACHE_SLABS(DT) \
-  ACACHE_CASE(DT, 4) ACACHE_CASE(DT, 2) ACACHE_CASE(DT, 1) ACACHE_CASE(DT, 3) \
-  ACACHE_CASE(DT, 5) ACACHE_CASE(DT, 6) ACACHE_CASE(DT, 7) ACACHE_CASE(DT, 8)
-  ACACHE_SLABS(ACACHE_BF16)
-  ACACHE_SLABS(ACACHE_F16)
-#undef ACACHE_SLABS
+#define ACACHE_DIMS(DT)                                                                             \
+  ACACHE_CASE(DT, 128) ACACHE_CASE(DT, 64) ACACHE_CASE(DT, 16) ACACHE_CASE(DT, 32) ACACHE_CASE(DT, 48)   \
+  ACACHE_CASE(DT, 80) ACACHE_CASE(DT, 96) ACACHE_CASE(DT, 112) ACACHE_CASE(DT, 144) ACACHE_CASE(DT, 160) \
+  ACACHE_CASE(DT, 176) ACACHE_CASE(DT, 192) ACACHE_CASE(DT, 208) ACACHE_CASE(DT, 224) ACACHE_CASE(DT, 240) \
+  ACACHE_CASE(DT, 256)
+  ACACHE_DIMS(ACACHE_BF16)
+  ACACHE_DIMS(ACACHE_F16)
+#undef ACACHE_DIMS
 #undef ACACHE_CASE
   return fail(ACACHE_E_SHAPE, "affix_importance: unsupported dtype / head_dim");
 }

@@ -65,7 +65,7 @@ def test_mask_rows_outside_q_are_absent_queries(device):
         cu_bad = torch.tensor([0, 23, 29], dtype=torch.int32)
         got = torch.zeros_like(clean)
         ops.affix_importance(got, q.to(device), kc.to(device), bad.to(device), cu_bad.to(device), 90, 23, **args)
-        assert torch.allclose(got, clean, rtol=1e-6, atol=1e-6)   # same rows, another tiling of them
+        assert torch.allclose(got, clean, rtol=1e-5, atol=1e-6)   # same rows, another tiling of them
 
 
 def test_argument_errors(device):

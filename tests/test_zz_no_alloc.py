@@ -57,7 +57,7 @@ def test_oversized_call_is_rejected_before_any_launch(device):
     q, kc, rows, cu, A, max_rows, kw = _inputs(device, 4, 4, 128, 50, [4], None, 4)
     imp = torch.zeros(1, A, dtype=torch.float32, device=device)
     # claim more mask rows than the array can keep statistics for: rejected from the sizes alone
-    too_many = limit // (4 * 8) + 1
+    too_many = limit // (4 * 4) + 1   # 4 heads x one fp32 statistic per mask row
     rc = lib.acache_affix_importance_noalloc(
         imp.data_ptr(), q.data_ptr(), kc.data_ptr(), rows.data_ptr(), cu.data_ptr(), None, None, None, 0,
         float(128 ** -0.5), A, 0, 1, q.shape[0], too_many, 4, 4, 4, 128, 0, kc.shape[0], imp.stride(0), q.stride(0), q.stride(1),
