@@ -167,6 +167,55 @@ def test_full_recomputation_matches_baseline_for_all_affix_layouts(device, token
 
 
 @pytest.mark.parametrize("max_num_seqs", [4, 1])
+def test_full_recomputation_matches_baseline_at_llada_head_geometry(device, max_num_seqs):
+    """The same invariant at the real attention geometry: 32 heads of 128 (d_model 4096), 256-token cache blocks,
+    a 300-token infix affix that crosses a cache block, a 32-token generation block; two layers keep it small.
+    Exercises the head-dim-128 attention, fused rotary + scatter and relocation kernels inside the engine."""
+    torch.manual_seed(11)
+    mask = 511
+    cfg = LLaDAConfig(vocab_size=512, d_model=4096, n_heads=32, n_layers=2, mlp_hidden_size=512,
+                      max_sequence_length=1024, mask_token_id=mask, rope_theta=500000.0)
+    model = LLaDAModelLM(cfg, init_std=0.02).to(device=device, dtype=torch.bfloat16).eval()
+    g = torch.Generator().manual_seed(5)
+    draw = lambda n: torch.randint(2, 500, (n,), generator=g).tolist()
+    head, affix, tail = draw(40), draw(300), draw(30)
+    tokens, a0, a1 = head + affix + tail, 40, 340
+
+    def serve(enable):
+        return Config(hf_config=cfg, mask_id=mask, recompute_batch_size=1, gen_length=32, block_length=32,
+                      cache_block_size=256, num_kvcache_blocks=10, temperature=0.0, threshold=0.0,
+                      enable_acache=enable, anchor_ratio=1.0, selection_mode="top", max_num_seqs=max_num_seqs)
+
+    def make():
+        return Sequence(tokens, gen_length=32, block_length=32, cache_block_size=256, mask_id=mask,
+                        prompt_affix_start=a0, prompt_affix_end=a1)
+
+    with torch.inference_mode():
+        base = ModelRunner(model, serve(False))
+        bseq = make()
+        base.block_manager.allocate(bseq)
+        bseq.finalize_slot_mapping()
+        ids, pos, _, _ = base.prepare_caching([bseq])
+        base_logits = model(ids, position_ids=pos).logits.float()
+        reset_context()
+
+        ac = ModelRunner(model, serve(True))
+        aseq = make()
+        affix_tokens = ac._prepare_acache([aseq])
+        ac._precompute_shared_prefix(list(affix_tokens))
+        aseq.set_anchor_positions(list(range(a0, a1)))
+        ac._reserve_single_sequence_relocation_workspace(aseq)
+        ac.block_manager.allocate(aseq)
+        ac._finalize_sequence_layout(aseq)
+        ids, pos, _ = ac.prepare_caching_acache([aseq])
+        ac_logits = model(ids, position_ids=pos).logits.float()
+        reset_context()
+    assert ac.shared_prefix_blocks == 2 and aseq.recompute_positions == list(range(len(aseq)))
+    assert float(base_logits.abs().max()) > 0.5          # the comparison is not between two all-zero tensors
+    torch.testing.assert_close(ac_logits, base_logits, rtol=5e-2, atol=5e-2)
+
+
+@pytest.mark.parametrize("max_num_seqs", [4, 1])
 def test_partial_anchor_refresh_matches_dense_recompute_of_the_same_layout(device, max_num_seqs):
     """anchor_ratio < 1: refresh logits must equal a dense forward in which the non-anchor affix keys are the
     cached shared keys moved to the request's positions — the semantics of affix reuse, for any relocation mode."""

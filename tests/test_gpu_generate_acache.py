@@ -1,4 +1,6 @@
 """Batch-1 entry points with the HF path's signatures (llada/generate_ACache.py) on the paged engine."""
+from pathlib import Path
+
 import pytest
 import torch
 
@@ -20,6 +22,58 @@ def _model(device, seed=0):
         model.model.transformer["ff_out"].weight[MASK].zero_()
         model.model.transformer["ff_out"].weight[0] += 0.05
     return cfg, model
+
+
+FIXTURE = Path(__file__).resolve().parent / "golden" / "hf_path_vectors.pt"
+
+
+def _fixture(device):
+    """The reference's own outputs (tests/golden/make_hf_path_vectors.py ran llada/generate_ACache.py on the CPU in
+    fp32 over a 2-layer random model with 2 heads of 128) and this package's model loaded with the same weights."""
+    data = torch.load(FIXTURE, weights_only=True)
+    model = LLaDAModelLM(LLaDAConfig(**data["config"]))
+    model.load_state_dict(data["weights"])       # same parameter names as the reference's LLaDAModelLM
+    return data["cases"], model.to(device=device, dtype=torch.bfloat16).eval()
+
+
+def test_importance_matches_the_reference_fixture(device):
+    """compute_attention_importance_cross_affix against the values the reference returned for prefix, infix and
+    suffix placement.  The reference ran in fp32, the engine in bf16 with the relocation on the query side:
+    measured difference 0.044 absolute / 4.6 % relative at most; bound 0.1 / 8 %.  The anchors chosen from the two
+    importance vectors must be the same tokens."""
+    cases, model = _fixture(device)
+    for c in cases:
+        kw = c["kwargs"]
+        cache = tuple((k.to(device), v.to(device)) for k, v in c["affix_cache"])
+        got = G.compute_attention_importance_cross_affix(model, c["masked_input"].to(device), cache, mask_id=MASK,
+                                                         affix_start=kw["affix_start"]).cpu()
+        want = c["importance"]
+        assert got.shape == want.shape
+        torch.testing.assert_close(got, want, rtol=8e-2, atol=1e-1, msg=lambda m: f"{c['name']}: {m}")
+        k = G.ceil_to_int(kw["anchor_ratio"] * want.shape[1])
+        assert G.select_anchor_tokens(got, k, "top").tolist() == G.select_anchor_tokens(want, k, "top").tolist(), c["name"]
+
+
+@pytest.mark.parametrize("from_cache", [True, False])
+def test_generation_matches_the_reference_fixture(device, from_cache):
+    """generate_with_anchor_attention against the reference's returned sequence and forward count, with the HF-layout
+    affix cache the reference was given and with the engine's own affix precompute.  Prompt positions and the
+    number of forwards must be equal; of the 8 generated tokens at most one may differ (fp32 there, bf16 here: an
+    arg-max near a tie can flip; measured: none differs)."""
+    cases, model = _fixture(device)
+    for c in cases:
+        kw = dict(c["kwargs"])
+        cache = tuple((k.to(device), v.to(device)) for k, v in c["affix_cache"]) if from_cache else None
+        x, nfe = G.generate_with_anchor_attention(model, c["prompt"].to(device), precomputed_affix_cache=cache, **kw)
+        want = c["x"]
+        assert nfe == c["nfe"] and x.shape == want.shape, c["name"]
+        start = kw.get("generation_start", c["prompt"].shape[1])
+        window = slice(start, start + kw["gen_length"])
+        outside = torch.ones(want.shape[1], dtype=torch.bool)
+        outside[window] = False
+        assert torch.equal(x.cpu()[0, outside], want[0, outside]), c["name"]
+        assert int((x.cpu()[0, window] != want[0, window]).sum()) <= 1, (c["name"], x[0, window].tolist(), want[0, window].tolist())
+        assert (x[0, window] != MASK).all()
 
 
 def test_helpers_match_the_reference_definitions(device):

@@ -115,24 +115,27 @@ def test_empty_input(device):
 
 
 def test_cpu_reference_config_fp32_llada_layer_shape(device):
-    """One layer slice of the fp32 configuration: A=512 affix rows moved to rows 384..895, shift +384,
-    theta 5e5, identity block table, 256-token blocks; 384 private request rows in further blocks."""
+    """The fp32 configuration at its full size: 32 layers x 32 KV heads x 128, A = 512 affix rows moved to rows
+    384..895 (shift +384, theta 5e5), identity block table, 256-token blocks, 384 private request rows in further
+    blocks.  One launch over all layers on the device, checked bit for bit against the oracle four layers at a time."""
     g = torch.Generator().manual_seed(0)
-    L, H, D, A, shift, BS = 2, 32, 128, 512, 384, 256
+    L, H, D, A, shift, BS = 32, 32, 128, 512, 384, 256
     nblocks = 4
     k = torch.randn(L, nblocks, BS, H, D, generator=g)
     v = torch.randn(L, nblocks, BS, H, D, generator=g)
     cos, sin = O.rope_table(896, D, 5e5)
     slot = torch.cat([torch.arange(2 * BS, 2 * BS + 384), torch.arange(A)]).to(torch.int32)
     delta = torch.cat([torch.zeros(384), torch.full((A,), shift)]).to(torch.int32)
-    ek, ev = O.relocate_rope_gather(k, v, slot, delta, cos, sin)
     gk, gv = ops.relocate_rope_gather(k.to(device), v.to(device), slot.to(device), delta.to(device),
                                       cos.to(device), sin.to(device))
     assert gk.shape == (L, 896, H, D)
-    assert torch.equal(_bits(gk.cpu()), _bits(ek))
-    assert torch.equal(_bits(gv.cpu()), _bits(ev))
+    gk, gv = gk.cpu(), gv.cpu()
+    for l in range(0, L, 4):
+        ek, ev = O.relocate_rope_gather(k[l:l + 4], v[l:l + 4], slot, delta, cos, sin)
+        assert torch.equal(_bits(gk[l:l + 4]), _bits(ek)), f"keys, layers {l}..{l + 3}"
+        assert torch.equal(_bits(gv[l:l + 4]), _bits(ev)), f"values, layers {l}..{l + 3}"
     # closed form: norms of (d, d+64) pairs survive the move
-    n0 = ek[:, 384:, :, :64] ** 2 + ek[:, 384:, :, 64:] ** 2
+    n0 = gk[:, 384:, :, :64] ** 2 + gk[:, 384:, :, 64:] ** 2
     n1 = k.reshape(L, -1, H, D)[:, :A, :, :64] ** 2 + k.reshape(L, -1, H, D)[:, :A, :, 64:] ** 2
     torch.testing.assert_close(n0, n1, atol=1e-4, rtol=1e-5)
 

@@ -69,7 +69,7 @@ def test_anchor_config_topk_then_scatter_all_layers(device):
         assert low[cu_k[b]:cu_k[b + 1]].tolist() == O.topk_anchors(w["scores"][b], w["K"][b], largest=False)
 
     # scatter the recomputed anchor rows of all layers into the first K_b private slots of each request
-    L, H, D, BS = 4, 4, 128, 256
+    L, H, D, BS = 28, 4, 128, 256                       # every layer of the Dream shape, one launch
     nblk = [-(-(k + r) // BS) for k, r in zip(w["K"], w["R"])]
     pool = torch.randperm(sum(nblk) + 8, generator=torch.Generator().manual_seed(1)) + 5
     slots, off = [], 0
