@@ -33,7 +33,7 @@ import torch
 
 from . import ops
 from .block_manager import BlockManager
-from .sequence import Sequence
+from .sequence import DeviceLayout, Sequence
 from .utils import add_gumbel_noise, get_context, reset_context, set_context
 
 
@@ -364,15 +364,27 @@ class ModelRunner:
         ascending, plus ``affix_start`` are the anchors (model_runner.py:833-843; ties go
         to the lower index).  One radix-select launch serves the whole batch.
         """
-        result = [[] for _ in seqs]
+        chosen, counts = self._select_anchors_on_device(seqs)
+        if chosen is None:
+            return [[] for _ in seqs]
+        flat, out, o = chosen.tolist(), [], 0
+        for k in counts:
+            out.append(flat[o:o + k])
+            o += k
+        return out
+
+    def _select_anchors_on_device(self, seqs: list[Sequence]):
+        """The same selection without the read-back: ``(anchors, counts)`` with ``anchors`` an int32 device tensor
+        holding every request's ascending anchor positions back to back and ``counts`` the number per request
+        (0 for a request without anchors); ``(None, counts)`` when no request has any."""
+        counts = [0] * len(seqs)
         active = [(i, s) for i, s in enumerate(seqs) if s.acache_enabled and s.num_anchor_tokens > 0]
         if not active:
-            return result
-        active_idx = [i for i, _ in active]
+            return None, counts
         active_seqs = [s for _, s in active]
         affix_len = active_seqs[0].affix_len
         if affix_len <= 0:
-            return result
+            return None, counts
         if any(s.affix_len != affix_len for s in active_seqs):
             raise ValueError("Batched Anchor Selection requires a consistent explicit prefix affix length.")
         importance = self._compute_affix_importance(active_seqs)
@@ -384,11 +396,11 @@ class ModelRunner:
         chosen = ops.topk_anchors(
             importance.view(-1), self._to_device(cu_a, torch.int32), self._to_device(cu_k, torch.int32),
             int(cu_k[-1]), offsets=self._to_device([s.affix_start for s in active_seqs], torch.int32),
-            largest=self.config.selection_mode != "bottom").tolist()
-        for b, i in enumerate(active_idx):
-            result[i] = chosen[cu_k[b]:cu_k[b + 1]]
+            largest=self.config.selection_mode != "bottom", out_dtype=torch.int32)
+        for (i, _), k in zip(active, ks):
+            counts[i] = k
         self._finish_timing(timing, "anchor_selection_topk", start)
-        return result
+        return chosen, counts
 
     def _compute_affix_importance(self, active_seqs: list[Sequence]) -> torch.Tensor:
         """fp32 ``[B, A]`` influence of every shared affix token on each request's [MASK] queries.
@@ -556,8 +568,18 @@ class ModelRunner:
             while True:
                 group = seqs[done:done + width]
                 try:
-                    for seq, anchors in zip(group, self._compute_anchor_positions_batch(group)):
-                        seq.set_anchor_positions(anchors)
+                    if self._device_layouts():
+                        chosen, counts = self._select_anchors_on_device(group)
+                        at = 0
+                        for seq, k in zip(group, counts):
+                            if seq.acache_enabled:
+                                seq.set_anchor_positions_on_device(chosen[at:at + k] if k else None)
+                            else:
+                                seq.set_anchor_positions([])
+                            at += k
+                    else:
+                        for seq, anchors in zip(group, self._compute_anchor_positions_batch(group)):
+                            seq.set_anchor_positions(anchors)
                     done += width
                     break
                 except torch.OutOfMemoryError as oom:
@@ -614,16 +636,66 @@ class ModelRunner:
             return 0
         self._prepare_admitted_sequences_for_acache(new_prompts, prefix_token_ids, allow_kv_cache_resize)
         self._reserve_single_sequence_relocation_workspace(new_prompts[0])
-        admitted = 0
+        admitted, on_device = 0, []
         for seq in new_prompts:
             if not self.block_manager.can_allocate(seq):
                 break
             self.block_manager.allocate(seq)
             self._record_kv_cache_usage(self._active_timing)
-            self._finalize_sequence_layout(seq)
+            if self._device_layouts() and seq.acache_enabled:
+                on_device.append(seq)
+            else:
+                self._finalize_sequence_layout(seq)
             batched_prompts.append(seq)
             admitted += 1
+        if on_device:
+            self._finalize_layouts_on_device(on_device)
         return admitted
+
+    def _device_layouts(self) -> bool:
+        """Slot maps and anchors stay on the device for batched serving.  The single-request mode
+        (``max_num_seqs == 1``) edits its read map on the host when it materialises the relocated affix, and the
+        HF-signature entry points run in that mode, so it keeps the host lists."""
+        return self.device.type == "cuda" and self.config.max_num_seqs != 1
+
+    def _finalize_layouts_on_device(self, seqs: list[Sequence]):
+        """``finalize_slot_mapping`` for all newly admitted requests in one launch, fed by the anchors that the
+        top-k launch left on the device (model_runner.py:833-843 reads them back with ``tolist`` and
+        sequence.py:169-202 loops over tokens on the host).  Also prepares, once per request, what every later
+        refresh would otherwise rebuild: the read map with the shared affix slots packed first (the order
+        query-side relocation wants, model_runner.py:275-282) and a device copy of the token ids."""
+        lengths = [len(s) for s in seqs]
+        counts = [s.num_anchor_tokens for s in seqs]
+        pending = [s.pending_device_anchors for s in seqs]
+        assert all((p is not None and p.numel() == k) or k == 0 for p, k in zip(pending, counts))
+        anchors = [p for p, k in zip(pending, counts) if k > 0]
+        anchors = (torch.cat(anchors) if len(anchors) > 1 else anchors[0]) if anchors else \
+            torch.zeros(0, dtype=torch.int32, device=self.device)
+        tables = self.prepare_block_tables(seqs)
+        read, rpos, rslot, cu_len, cu_rec = ops.build_slot_layout(
+            lengths, [(s.affix_start, s.affix_end) for s in seqs], anchors, tables, self.config.cache_block_size,
+            0, anchor_counts=counts)
+        uses_rope = bool(getattr(self.config.hf_config, "rope", True))
+        moved = [uses_rope and s.affix_start != 0 for s in seqs]
+        packed = None
+        if any(moved):
+            # stable partition inside each request: shared affix slots (0 .. shared_prefix_len) first
+            seg = np.repeat(np.arange(len(seqs), dtype=np.int64), lengths)
+            flag = self._to_device(np.repeat(np.asarray(moved), lengths), torch.bool)
+            private = ~((read >= 0) & (read < self.shared_prefix_len) & flag)
+            order = torch.argsort(self._to_device(seg * 2, torch.int64) + private, stable=True)
+            packed = read[order]
+        tokens = self._to_device(np.concatenate([np.asarray(s.token_ids, dtype=np.int64) for s in seqs]), torch.int64)
+        rpos64 = rpos.to(torch.int64)
+        at = 0
+        for b, seq in enumerate(seqs):
+            lo, hi, r0, r1 = cu_len[b], cu_len[b + 1], cu_rec[b], cu_rec[b + 1]
+            seq.attach_device_layout(DeviceLayout(
+                anchors[at:at + counts[b]], read[lo:hi], packed[lo:hi] if moved[b] else None,
+                rpos64[r0:r1], rslot[r0:r1], tokens[lo:hi]))
+            seq.pending_device_anchors = None
+            seq.relocated_affix_materialized = False
+            at += counts[b]
 
     # ------------------------------------------------------------------ context builders (1004-1114, 1295-1471)
     def _select(self, seqs, active_indices):
@@ -679,6 +751,8 @@ class ModelRunner:
         """Cache refresh with affix reuse: queries = anchors + non-affix tokens; keys read through ``read_slot_map``."""
         group = self._select(seqs, active_indices)
         self._configure_affix_relocation(group)
+        if use_query_relocation is None and all(s.device_layout is not None for s in group):
+            return self._prepare_caching_from_device_layouts(group)
         relocation_materialized = all(getattr(s, "relocated_affix_materialized", False) for s in group)
         if use_query_relocation is None:
             use_query_relocation = self.config.max_num_seqs != 1
@@ -712,11 +786,75 @@ class ModelRunner:
         return (self._to_device(np.concatenate(ids), torch.int64), self._to_device(np.concatenate(pos), torch.int64),
                 self._to_device(block_starts, torch.int32))
 
+    def _device_read_side(self, group):
+        """Per request: the read map in the order attention wants it and the number of shared slots in front
+        (the device twin of ``_attention_read_layout``); plus the metadata tensors both context builders share."""
+        packed = self._affix_relocation_enabled   # batched serving never materialises: query-side relocation
+        reads, shared_lens, cu_k = [], [], [0]
+        for seq in group:
+            layout = seq.device_layout
+            if packed and layout.read_packed is not None:
+                reads.append(layout.read_packed)
+                shared_lens.append(seq.affix_len - seq.num_anchor_tokens)
+            else:
+                reads.append(layout.read)
+                shared_lens.append(0)
+            cu_k.append(cu_k[-1] + len(seq))
+        shifts = [seq.affix_start if self._affix_relocation_enabled else 0 for seq in group]
+        return packed, reads, shared_lens, shifts, cu_k
+
+    def _context_metadata(self, *rows):
+        """Several short int32 host lists in one pinned buffer and one copy; returns the device slices."""
+        sizes = [len(r) for r in rows]
+        flat = self._to_device(np.concatenate([np.asarray(r, dtype=np.int64) for r in rows]), torch.int32)
+        out, at = [], 0
+        for n in sizes:
+            out.append(flat[at:at + n])
+            at += n
+        return out
+
+    def _prepare_caching_from_device_layouts(self, group):
+        """``prepare_caching_acache`` when the requests' slot maps live on the device: a few concatenations of
+        per-request tensors and one small metadata copy; no per-token host work, no read-back."""
+        packed, reads, shared_lens, shifts, cu_k = self._device_read_side(group)
+        layouts = [s.device_layout for s in group]
+        n_rec = [s.num_anchor_tokens + len(s) - s.affix_len for s in group]
+        cu_q = [0] + list(np.cumsum(n_rec))
+        block_starts = [cu_q[b] + s.block_query_start() for b, s in enumerate(group)]
+        kv_lens = np.diff(cu_k)
+        d_cu_q, d_cu_k, d_kv, d_shared, d_shifts, d_starts = self._context_metadata(
+            cu_q, cu_k, kv_lens, shared_lens, shifts, block_starts)
+        positions = torch.cat([l.recompute_pos for l in layouts])
+        input_ids = torch.cat([l.tokens.index_select(0, l.recompute_pos) for l in layouts])
+        set_context(
+            True, d_cu_q, d_cu_k, d_kv, int(max(n_rec)), int(kv_lens.max()),
+            torch.cat([l.recompute_slots for l in layouts]), None, True, torch.cat(reads),
+            d_shared if packed else None, d_shifts, total_k=int(cu_k[-1]))
+        return input_ids, positions, d_starts
+
+    def _prepare_decoding_from_device_layouts(self, group):
+        """``prepare_decoding_acache`` from the device layouts: the current block's slots are a slice of each
+        request's read map."""
+        block_length = self.config.block_length
+        packed, reads, shared_lens, shifts, cu_k = self._device_read_side(group)
+        starts = [s.generation_start + s.current_block_idx * block_length for s in group]
+        kv_lens = np.diff(cu_k)
+        cu_q = np.arange(len(group) + 1) * block_length
+        d_cu_q, d_cu_k, d_kv, d_shared, d_shifts = self._context_metadata(cu_q, cu_k, kv_lens, shared_lens, shifts)
+        slots = torch.cat([s.device_layout.read[b0:b0 + block_length] for s, b0 in zip(group, starts)])
+        positions = np.asarray(starts, dtype=np.int64)[:, None] + np.arange(block_length)[None, :]
+        set_context(
+            False, d_cu_q, d_cu_k, d_kv, block_length, int(kv_lens.max()), slots, None, True, torch.cat(reads),
+            d_shared if packed else None, d_shifts, total_k=int(cu_k[-1]))
+        return self._to_device(positions, torch.int64)
+
     def prepare_decoding_acache(self, seqs, active_indices=None):
         """Block refinement with affix reuse: the current block's tokens against the same read slot maps."""
         group = self._select(seqs, active_indices)
         block_length = self.config.block_length
         self._configure_affix_relocation(group)
+        if all(s.device_layout is not None for s in group):
+            return self._prepare_decoding_from_device_layouts(group)
         relocation_materialized = all(getattr(s, "relocated_affix_materialized", False) for s in group)
         use_query_relocation = self._use_query_side_affix_relocation(relocation_materialized)
         starts, slots, reads, shared_lens, shifts, cu_k = [], [], [], [], [], [0]
@@ -836,6 +974,7 @@ class ModelRunner:
                 self._finish_timing(timing, "cache_forward", start)
                 self._add_timing_count(timing, "cache_forward_calls", 1)
                 self._add_timing_count(timing, "cache_forward_nfe", len(part))
+                self._add_timing_count(timing, "cache_forward_tokens", int(input_ids.numel()))
                 start = self._start_timing()
                 logits = logits.view(len(part), block_length, -1)
                 if dream:
@@ -874,6 +1013,8 @@ class ModelRunner:
                     seq = batch[row]
                     begin = seq.generation_start + seq.current_block_idx * block_length
                     seq.token_ids[begin:begin + block_length] = working[row].tolist()
+                    if seq.device_layout is not None:
+                        seq.device_layout.tokens[begin:begin + block_length] = working[row]
                     seq.current_block_idx += 1
                     if seq.current_block_idx >= seq.num_blocks_to_generate:
                         self.block_manager.deallocate(seq)
@@ -929,6 +1070,7 @@ class ModelRunner:
                 self._finish_timing(timing, "decode_forward", start)
                 self._add_timing_count(timing, "decode_forward_calls", 1)
                 self._add_timing_count(timing, "decode_forward_nfe", len(active))
+                self._add_timing_count(timing, "decode_forward_tokens", len(active) * block_length)
                 start = self._start_timing()
                 current_blocks = working[active]
                 x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,

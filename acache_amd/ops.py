@@ -383,23 +383,27 @@ def affix_importance_workspace_bytes(total_mask_rows: int, batch: int, num_heads
 
 
 def build_slot_layout(lengths, affix_spans, anchors, block_tables: torch.Tensor, block_size: int,
-                      shared_slot_offset: int = 0):
+                      shared_slot_offset: int = 0, anchor_counts=None):
     """Read slot maps and recompute lists of a batch in one launch (``Sequence.finalize_slot_mapping``,
     nano-vdllm/sequence.py:169-202, for every request at once).
 
     ``lengths``: tokens per request; ``affix_spans``: ``(start, end)`` per request; ``anchors``: ascending anchor
-    positions per request; ``block_tables``: int32 ``[B, max_blocks]`` on the device (-1 padded).
+    positions per request as lists, or — with ``anchor_counts`` giving the number per request — one int32 device
+    tensor holding them back to back (the output of ``topk_anchors``, which then never visits the host);
+    ``block_tables``: int32 ``[B, max_blocks]`` on the device (-1 padded).
     Returns ``(read_slots, recompute_pos, recompute_slots, cu_len, cu_rec)``, the first three int32 device tensors.
     """
     device = block_tables.device
     B = len(lengths)
     assert block_tables.is_cuda and block_tables.dtype == torch.int32 and block_tables.is_contiguous()
-    assert block_tables.shape[0] == B == len(affix_spans) == len(anchors)
-    rec = [len(a) + n - (e - s) for n, (s, e), a in zip(lengths, affix_spans, anchors)]
+    on_device = anchor_counts is not None
+    counts = [int(c) for c in anchor_counts] if on_device else [len(a) for a in anchors]
+    assert block_tables.shape[0] == B == len(affix_spans) == len(counts)
+    rec = [k + n - (e - s) for n, (s, e), k in zip(lengths, affix_spans, counts)]
     cu_len = [0] + list(_accumulate(lengths))
     cu_rec = [0] + list(_accumulate(rec))
-    cu_anc = [0] + list(_accumulate(len(a) for a in anchors))
-    flat_anchors = [p for a in anchors for p in a]
+    cu_anc = [0] + list(_accumulate(counts))
+    flat_anchors = [] if on_device else [p for a in anchors for p in a]
     meta = torch.tensor(cu_len + cu_rec + cu_anc + [s for s, _ in affix_spans] + [e for _, e in affix_spans]
                         + (flat_anchors or [0]), dtype=torch.int32).to(device, non_blocking=True)
     o = 0
@@ -408,6 +412,9 @@ def build_slot_layout(lengths, affix_spans, anchors, block_tables: torch.Tensor,
         parts.append(meta[o:o + n])
         o += n
     d_len, d_rec, d_anc, d_start, d_end, d_anchors = parts
+    if on_device and cu_anc[-1] > 0:
+        d_anchors = _i32(anchors, "anchors")
+        assert d_anchors.is_cuda and d_anchors.numel() == cu_anc[-1]
     read = torch.empty(cu_len[-1], dtype=torch.int32, device=device)
     rpos = torch.empty(cu_rec[-1], dtype=torch.int32, device=device)
     rslot = torch.empty(cu_rec[-1], dtype=torch.int32, device=device)

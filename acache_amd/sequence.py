@@ -27,8 +27,49 @@ class SequenceStatus(Enum):
     FINISHED = auto()
 
 
+class DeviceLayout:
+    """Slot maps of one request as device tensors (views into the tensors the layout kernel filled for a whole
+    admission batch), for an engine that never brings them to the host.
+
+    ``anchors`` int32 ascending anchor positions; ``read`` int32 read slot per logical position; ``read_packed`` the
+    same slots with the shared affix slots moved to the front (query-side relocation order) or ``None``;
+    ``recompute_pos`` int64 / ``recompute_slots`` int32: the rows a cache refresh recomputes and where their K/V
+    go; ``tokens`` int64 token ids, kept current by the engine as blocks are committed."""
+
+    __slots__ = ("anchors", "read", "read_packed", "recompute_pos", "recompute_slots", "tokens")
+
+    def __init__(self, anchors, read, read_packed, recompute_pos, recompute_slots, tokens):
+        self.anchors, self.read, self.read_packed = anchors, read, read_packed
+        self.recompute_pos, self.recompute_slots, self.tokens = recompute_pos, recompute_slots, tokens
+
+
+def _host_mirror(name: str, fetch):
+    """A list-valued attribute that may live on the device: read back (and kept) the first time the host asks."""
+    slot = "_" + name
+
+    def get(self):
+        value = self.__dict__.get(slot)
+        if value is None:
+            value = fetch(self)
+            self.__dict__[slot] = value
+        return value
+
+    def put(self, value):
+        self.__dict__[slot] = value
+
+    return property(get, put)
+
+
 class Sequence:
     counter = itertools.count()
+
+    # host lists of the reference; with a device layout attached they are fetched on first use only
+    anchor_positions = _host_mirror(
+        "anchor_positions", lambda s: (s.device_layout.anchors if s.device_layout is not None
+                                       else s.pending_device_anchors).tolist())
+    recompute_positions = _host_mirror("recompute_positions", lambda s: s.device_layout.recompute_pos.tolist())
+    recompute_slot_mapping = _host_mirror("recompute_slot_mapping", lambda s: s.device_layout.recompute_slots.tolist())
+    read_slot_map = _host_mirror("read_slot_map", lambda s: s.device_layout.read.tolist())
 
     def __init__(
         self,
@@ -82,6 +123,8 @@ class Sequence:
         self.num_blocks_to_generate = -(-gen_length // block_length)
 
         self.acache_enabled = False
+        self.device_layout: DeviceLayout | None = None
+        self.pending_device_anchors = None   # anchors chosen on the device, before blocks are allocated
         self.affix_start, self.affix_end = a0, a1
         self.affix_len = 0
         self.anchor_positions: list[int] = []
@@ -168,6 +211,8 @@ class Sequence:
         self.affix_len = a1 - a0
         self.acache_enabled = self.affix_len > 0
         self.num_anchor_tokens = min(math.ceil(anchor_ratio * self.affix_len), self.affix_len)
+        self.device_layout = None
+        self.pending_device_anchors = None
         self.anchor_positions = []
         self.recompute_positions = list(range(self.num_tokens))
         self.recompute_slot_mapping = []
@@ -187,6 +232,22 @@ class Sequence:
         self.anchor_positions = chosen
         self.num_anchor_tokens = len(chosen)
         self.recompute_positions = sorted(chosen + self.non_affix_positions)
+
+    def set_anchor_positions_on_device(self, anchors):
+        """The engine's top-k left this request's ascending anchor positions in a device tensor (``None`` for a
+        request without anchors); ``anchor_positions`` reads them back only if somebody asks."""
+        assert self.acache_enabled
+        self.pending_device_anchors = anchors
+        self.anchor_positions = None if anchors is not None else []
+
+    def attach_device_layout(self, layout: DeviceLayout, shared_slot_offset: int = 0):
+        """The engine built this request's anchors and slot maps on the device (top-k and the layout kernel):
+        adopt them without a read-back.  The four host lists are fetched from the tensors if anybody asks."""
+        assert self.acache_enabled and layout.anchors.numel() == self.num_anchor_tokens
+        self.device_layout = layout
+        self.shared_slot_offset = shared_slot_offset
+        for name in ("anchor_positions", "recompute_positions", "recompute_slot_mapping", "read_slot_map"):
+            setattr(self, name, None)
 
     def private_slots(self) -> np.ndarray:
         """Slots owned by this request, block by block in ``block_table`` order."""
@@ -238,8 +299,13 @@ class Sequence:
         self.read_slot_map = read.tolist()
 
     def block_query_start(self):
+        """Index of the current block's first token among the recomputed rows (sequence.py:204-206 looks it up in
+        the list; anchors all lie inside the affix, so the index follows from the spans alone)."""
         start = self.generation_start + self.current_block_idx * self.block_length
-        return self.recompute_positions.index(start)
+        if not self.acache_enabled or start < self.affix_start:
+            return start
+        anchors = self.num_anchor_tokens if self.device_layout is not None else len(self.anchor_positions)
+        return start - self.affix_len + anchors
 
     def __getstate__(self):
         return (self.num_tokens, self.num_prompt_tokens, self.block_table)

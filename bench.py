@@ -3,9 +3,13 @@
 
 One "step" = one pass of relocate + RoPE re-rotate + gather over the ragged bf16
 batch of 16 LLaDA-8B-shaped requests, all 32 layers (one kernel launch), inputs
-resident in HBM.  The same run also times the anchor-recompute varlen attention
-(one layer call, reported under "attention") and the reference-style torch CPU
-formulation on a bounded sample (reported under "cpu_baseline").
+resident in HBM.  The same run also measures, each with its own workload, roofline
+and CPU baseline on a bounded sample:
+  "attention"              the anchor-recompute varlen attention, one layer call (configs[3]);
+  "relocate_fp32"          the fp32 single-request configuration, 32 layers (configs[0]);
+  "anchor_select_scatter"  one top-k launch + one 28-layer scatter launch, Dream shape (configs[2]);
+  "engine"                 full affix recompute vs anchor ratio 0.2 on random-init LLaDA-8B-shaped
+                           weights, 16 requests x 256 generated tokens (configs[4]).
 
 Prints ONE JSON line.  `python bench.py --gpus 1 --steps K --warmup W`.
 """
@@ -25,10 +29,13 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, vendor figure
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 
-# HBM bytes per launch of the default workloads, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script (raw counters scaled by what they read for the 1 GiB copy of --copy-calibration: x2.000 and x1.000);
-# the summaries with the commands are profiles/relocate_kernel_*.md and profiles/varlen_attn_dma_kernel_*.md.
-MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 18.029e9, "attention": 284.5e6}
+# HBM bytes per launch of the default workloads.  Not measured by this run: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this script (raw counters scaled by what they read for the 1 GiB copy of
+# --copy-calibration), taken at the commit named here; profiles/*.md hold the summaries and their commands.
+# A kernel changed after that commit makes its figure stale: re-run the counters and update both.
+MEASURED_TRAFFIC_COMMIT = "TRAFFIC_COMMIT_PLACEHOLDER"
+MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 18.029e9, "attention": 284.5e6, "relocate_fp32": None,
+                          "scatter_28_layers": None}
 
 
 def _event_times_ms(fn, steps, torch):
@@ -172,11 +179,161 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
                    "total_q": total_q, "total_kv": sum(w["kv_lens"])},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["attention"],
-                     "kernel": "varlen_attn_dma_kernel<bf16,128,plain>", "algorithmic_flops": flops,
+                     "kernel": "varlen_attn_unit_kernel<bf16,128,plain>", "algorithmic_flops": flops,
                      "algorithmic_bytes": kv_bytes + qo_bytes,
                      "achieved_GBps": round((kv_bytes + qo_bytes) / (avg_ms * 1e-3) / 1e9, 1),
                      "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)},
     }
+
+
+def _cpu_median_s(fn, runs=7, warm=2, budget_s=15.0):
+    times, t_begin = [], time.perf_counter()
+    for i in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        dt = time.perf_counter() - t0
+        if i >= warm:
+            times.append(dt)
+        if time.perf_counter() - t_begin > budget_s and times:
+            break
+    return statistics.median(times), len(times)
+
+
+def relocate_fp32_bench(torch, device, ops, steps, warmup, cpu_baseline=True):
+    """configs[0]: one request, fp32, 32 layers x 32 KV heads x 128; a 512-token affix cached at positions 0..511
+    moved behind 384 request rows (shift +384, theta 5e5), identity block table, packed [896, 32, 128] per layer.
+    Reported twice: the whole packed buffer (384 copied + 512 rotated rows) and the affix rows alone."""
+    from acache_amd.rope import rope_table
+    from oracle import acache_oracle as O
+
+    L, H, D, A, shift, BS, R = 32, 32, 128, 512, 384, 256, 384
+    gen = torch.Generator(device=device).manual_seed(0)
+    k = torch.randn(L, 4, BS, H, D, generator=gen, device=device)
+    v = torch.randn(L, 4, BS, H, D, generator=gen, device=device)
+    cos, sin = rope_table(A + shift, D, 5e5)
+    cos, sin = cos.to(device), sin.to(device)
+    slot = torch.cat([torch.arange(2 * BS, 2 * BS + R), torch.arange(A)]).to(torch.int32).to(device)
+    delta = torch.cat([torch.zeros(R), torch.full((A,), shift)]).to(torch.int32).to(device)
+    out_k = torch.empty(L, R + A, H, D, device=device)
+    out_v = torch.empty_like(out_k)
+
+    def whole():
+        ops.relocate_rope_gather(k, v, slot, delta, cos, sin, out_k=out_k, out_v=out_v)
+
+    def affix_only():
+        ops.relocate_rope_gather(k, v, slot[R:], delta[R:], cos, sin, out_k=out_k[:, :A], out_v=out_v[:, :A])
+
+    row = H * D * 4
+    res = {}
+    for name, fn, rows in (("whole_buffer", whole, R + A), ("affix_only", affix_only, A)):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        ms = _event_times_ms(fn, steps, torch)[0]
+        nbytes = 2 * 2 * rows * row * L + 8 * rows
+        res[name] = {"rows": rows, "ms_per_launch": round(ms, 4), "algorithmic_bytes": nbytes,
+                     "GBps": round(nbytes / ms / 1e6, 1)}
+    out = {
+        "metric": "affix KV relocate+RoPE GB/s, fp32", "unit": "GB/s", "value": res["whole_buffer"]["GBps"],
+        "dtype": "f32",
+        "config": {"workload": "configs[0]: 1 request, fp32, 32 layers x 32 KV heads x 128, affix 512 rows shifted by +384 "
+                               "behind 384 request rows, 256-token blocks, identity block table, packed [896, 32, 128] per layer"},
+        "whole_buffer": res["whole_buffer"], "affix_only": res["affix_only"],
+        "roofline": {"bound": "hbm", "achieved": res["whole_buffer"]["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(res["whole_buffer"]["GBps"] / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES["relocate_fp32"], "kernel": "relocate_kernel<f32,128>",
+                     "avg_launch_ms": res["whole_buffer"]["ms_per_launch"],
+                     "algorithmic_bytes": res["whole_buffer"]["algorithmic_bytes"]},
+    }
+    if cpu_baseline:
+        torch.set_num_threads(os.cpu_count() or 1)
+        layers = 2
+        ck, cv = k[:layers].cpu(), v[:layers].cpu()
+        cslot, cdelta, ccos, csin = slot.cpu(), delta.cpu(), cos.cpu(), sin.cpu()
+        med, n = _cpu_median_s(lambda: O.relocate_rope_gather(ck, cv, cslot, cdelta, ccos, csin), budget_s=10.0)
+        out["cpu_baseline"] = dict(value=round(2 * 2 * (R + A) * row * layers / med / 1e9, 2), unit="GB/s",
+                                   cores=torch.get_num_threads(), kind="port",
+                                   sample=f"{layers} of {L} layers of the same request (whole buffer), median of {n} runs after 2 warm-ups, {med * 1e3:.0f} ms each")
+    return out
+
+
+def anchor_select_scatter_bench(torch, device, ops, steps, warmup, cpu_baseline=True):
+    """configs[2]: Dream shape (28 layers, 4 KV heads, D 128, bf16), batch 16 with infix placement: one top-k launch
+    over the ragged influence scores (anchor ratio 0.2, 5 % injected ties) and one launch that scatters the
+    recomputed anchor K/V of all 28 layers back into the paged cache."""
+    from acache_amd.synthetic import anchor_batch
+
+    w = anchor_batch(seed=0)
+    L, Hkv, D, BS = 28, 4, 128, 256
+    n_anchor, n_scores = sum(w["K"]), sum(w["A"])
+    gen = torch.Generator(device=device).manual_seed(0)
+    nblk = sum(-(-k // BS) for k in w["K"]) + 2
+    key = torch.randn(L, n_anchor, Hkv, D, generator=gen, device=device).to(torch.bfloat16)
+    val = torch.randn(L, n_anchor, Hkv, D, generator=gen, device=device).to(torch.bfloat16)
+    kc = torch.zeros(L, nblk, BS, Hkv, D, dtype=torch.bfloat16, device=device)
+    vc = torch.zeros_like(kc)
+    slots = torch.randperm(nblk * BS, device=device)[:n_anchor].to(torch.int32)
+    scores = torch.cat(w["scores"]).to(device)
+    cu_a = torch.tensor([0] + np_cumsum(w["A"]), dtype=torch.int32, device=device)
+    cu_k = torch.tensor([0] + np_cumsum(w["K"]), dtype=torch.int32, device=device)
+    starts = torch.tensor(w["affix_start"], dtype=torch.int32, device=device)
+
+    def scatter():
+        ops.kv_scatter_layers(key, val, kc, vc, slots)
+
+    def topk():
+        ops.topk_anchors(scores, cu_a, cu_k, n_anchor, offsets=starts)
+
+    timed = {}
+    for name, fn in (("scatter", scatter), ("topk", topk)):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        timed[name] = _event_times_ms(fn, steps, torch)[0]
+    scatter_bytes = 2 * 2 * n_anchor * Hkv * D * 2 * L + 4 * n_anchor
+    topk_bytes = 4 * n_scores + 8 * n_anchor
+    gbps = scatter_bytes / timed["scatter"] / 1e6
+    out = {
+        "metric": "anchor top-k us; anchor K/V scatter GB/s", "unit": "GB/s", "value": round(gbps, 1), "dtype": "bf16",
+        "config": {"workload": f"configs[2]: Dream shape (28 layers, 4 KV heads, D 128, bf16), batch 16, infix placement, "
+                               f"{n_scores} fp32 influence scores with 5% ties, anchor ratio 0.2 -> {n_anchor} anchors, "
+                               f"their K/V rows of all 28 layers scattered into a paged cache of {nblk} blocks"},
+        "topk": {"us_per_launch": round(timed["topk"] * 1e3, 2), "algorithmic_bytes": topk_bytes,
+                 "GBps": round(topk_bytes / timed["topk"] / 1e6, 2), "kernel": "topk_kernel",
+                 "note": "81 KB of input: a latency-bound launch (16 workgroups), not a bandwidth figure"},
+        "scatter": {"us_per_launch": round(timed["scatter"] * 1e3, 2), "algorithmic_bytes": scatter_bytes,
+                    "GBps": round(gbps, 1), "kernel": "scatter_kernel<bf16>"},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES["scatter_28_layers"],
+                     "kernel": "scatter_kernel<bf16>", "avg_launch_ms": round(timed["scatter"], 5),
+                     "algorithmic_bytes": scatter_bytes,
+                     "note": "166 MB written over a 332 MB working set: smaller than the 256 MB last-level cache, so "
+                             "part of the traffic never reaches HBM"},
+    }
+    if cpu_baseline:
+        torch.set_num_threads(os.cpu_count() or 1)
+        cpu_scores = [t.clone() for t in w["scores"]]
+        ck, cv = key[0].cpu(), val[0].cpu()
+        ckc = torch.zeros(nblk * BS, Hkv, D, dtype=torch.bfloat16)
+        cvc = torch.zeros_like(ckc)
+        cslots = slots.cpu().long()
+
+        def cpu_topk():   # the reference's formulation: torch.topk + sort per request (model_runner.py:833-843)
+            return [torch.topk(sc, k).indices.sort().values + a0 for sc, k, a0 in zip(cpu_scores, w["K"], w["affix_start"])]
+
+        def cpu_scatter():
+            ckc.index_copy_(0, cslots, ck)
+            cvc.index_copy_(0, cslots, cv)
+
+        t_topk, n1 = _cpu_median_s(cpu_topk, budget_s=5.0)
+        t_scatter, n2 = _cpu_median_s(cpu_scatter, budget_s=5.0)
+        out["cpu_baseline"] = dict(
+            value=round(2 * 2 * n_anchor * Hkv * D * 2 / t_scatter / 1e9, 2), unit="GB/s", cores=torch.get_num_threads(),
+            kind="port", topk_us=round(t_topk * 1e6, 1),
+            sample=f"scatter: index_copy_ of K and V for 1 of 28 layers ({n_anchor} rows), median of {n2} runs, "
+                   f"{t_scatter * 1e6:.0f} us each; top-k: torch.topk + sort per request on the same scores, "
+                   f"median of {n1} runs, {t_topk * 1e6:.0f} us")
+    return out
 
 
 def attention_shape_sweep(torch, device, ops, steps):
@@ -328,6 +485,7 @@ def kernel_sweep(torch, device, ops, steps):
 
 
 def np_cumsum(values):
+    """Inclusive running sums as a list of Python ints."""
     total, acc = 0, []
     for v in values:
         total += int(v)
@@ -335,9 +493,56 @@ def np_cumsum(values):
     return acc
 
 
-def engine_bench(torch, device, args):
+def cpu_engine_baseline(torch, cfg, rows):
+    """Reference-style torch CPU formulation of ONE transformer layer (fp32: RMSNorm, q/k/v projections, rotary,
+    ``scaled_dot_product_attention`` over each request's keys, output projection, SwiGLU MLP) on the 512 query
+    tokens of one refinement step (16 requests x 32 tokens, 1 400 keys each).  Scaled to an engine rate by the
+    layer count and by the query tokens the GPU's ratio-0.2 run pushed through the model."""
+    import torch.nn.functional as F
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    d, h, m = cfg.d_model, cfg.n_heads, cfg.mlp_hidden_size
+    hd = d // h
+    g = torch.Generator().manual_seed(0)
+    w = {n: torch.randn(o, i, generator=g) * 0.02 for n, (o, i) in
+         dict(q=(d, d), k=(d, d), v=(d, d), o=(d, d), gate=(m, d), up=(m, d), down=(d, m)).items()}
+    B, Lq, Lk = 16, 32, 1400
+    x = torch.randn(B, Lq, d, generator=g)
+    kc = torch.randn(B, h, Lk, hd, generator=g)
+    vc = torch.randn(B, h, Lk, hd, generator=g)
+    cos = torch.randn(Lq, hd, generator=g)
+    sin = torch.randn(Lq, hd, generator=g)
+
+    def rot(t):
+        t1, t2 = t[..., : hd // 2], t[..., hd // 2:]
+        return t * cos + torch.cat([-t2, t1], dim=-1) * sin
+
+    def layer():
+        y = F.rms_norm(x, (d,))
+        q = rot(F.linear(y, w["q"]).view(B, Lq, h, hd).transpose(1, 2))
+        k = rot(F.linear(y, w["k"]).view(B, Lq, h, hd).transpose(1, 2))
+        v = F.linear(y, w["v"]).view(B, Lq, h, hd).transpose(1, 2)
+        kk = torch.cat([kc[:, :, : Lk - Lq], k], dim=2)
+        vv = torch.cat([vc[:, :, : Lk - Lq], v], dim=2)
+        a = F.scaled_dot_product_attention(q, kk, vv).transpose(1, 2).reshape(B, Lq, d)
+        z = x + F.linear(a, w["o"])
+        y2 = F.rms_norm(z, (d,))
+        return z + F.linear(F.silu(F.linear(y2, w["gate"])) * F.linear(y2, w["up"]), w["down"])
+
+    med, n = _cpu_median_s(layer, runs=5, warm=1, budget_s=15.0)
+    acache = next(r for r in rows if r["mode"].startswith("acache"))
+    tokens = acache["timing"].get("cache_forward_tokens", 0) + acache["timing"].get("decode_forward_tokens", 0)
+    est = tokens / (B * Lq) * med * cfg.n_layers
+    return dict(value=round(acache["generated_tokens"] / est, 2), unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"one of {cfg.n_layers} layers on the 512 query tokens of one refinement step, fp32, median of {n} runs, "
+                       f"{med * 1e3:.0f} ms; scaled by {cfg.n_layers} layers and the {tokens} query tokens of the GPU's "
+                       f"{acache['mode']} run (an extrapolation: the whole run on the host would take ~{est:.0f} s)")
+
+
+def engine_bench(torch, device, args, ratios=None, cpu_baseline=False):
     """configs[4]: nano-vdllm-style engine step on random-init LLaDA-8B-shaped weights, anchor-ratio sweep
-    against full affix recompute.  Prints one JSON line of its own (not part of the default run)."""
+    against full affix recompute.  Returns the result object (``--engine`` prints it as its own JSON line; the
+    default run embeds a two-mode version under "engine")."""
     import numpy as np
     from acache_amd import Config, Sequence
     from acache_amd.llada import LLaDAConfig, LLaDAModelLM
@@ -392,7 +597,8 @@ def engine_bench(torch, device, args):
     print("[engine] warm-up done", file=sys.stderr, flush=True)
 
     rows = []
-    for label, enable, ratio in [("full_recompute", False, 0.0)] + [(f"acache_{r}", True, r) for r in args.engine_ratios]:
+    ratios = args.engine_ratios if ratios is None else ratios
+    for label, enable, ratio in [("full_recompute", False, 0.0)] + [(f"acache_{r}", True, r) for r in ratios]:
         runner = ModelRunner(model, serve(enable, ratio))
         seqs = prompts()
         torch.cuda.synchronize()
@@ -401,7 +607,8 @@ def engine_bench(torch, device, args):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         tokens = sum(len(o) for o in out)
-        timing = {k: round(v, 4) for k, v in runner.last_timing.items() if isinstance(v, float)}
+        timing = {k: round(v, 4) if isinstance(v, float) else v for k, v in runner.last_timing.items()
+                  if isinstance(v, (int, float)) and not k.startswith("kv_cache_")}
         rows.append({"mode": label, "anchor_ratio": ratio, "seconds": round(dt, 3), "generated_tokens": tokens,
                      "tokens_per_s": round(tokens / dt, 1), "nfe": int(nfe), "timing": timing})
         print(f"[engine] {label}: {tokens / dt:.1f} tok/s, nfe {nfe}, {dt:.2f} s", file=sys.stderr, flush=True)
@@ -410,13 +617,29 @@ def engine_bench(torch, device, args):
     base = rows[0]["tokens_per_s"]
     for r in rows:
         r["speedup_vs_full_recompute"] = round(r["tokens_per_s"] / base, 3)
-    print(json.dumps({
-        "metric": "engine generated tokens/s vs full affix recompute", "unit": "tokens/s", "n_gpus": 1, "dtype": "bf16",
-        "data": "synthetic",
+        # matrix-product work of the forwards (projections, MLP, output head on the kept rows), attention excluded
+        tok = r["timing"].get("cache_forward_tokens", 0) + r["timing"].get("decode_forward_tokens", 0)
+        kept = (r["timing"].get("cache_forward_nfe", 0) + r["timing"].get("decode_forward_nfe", 0)) * block
+        per_token = 2 * cfg.n_layers * (4 * cfg.d_model ** 2 + 3 * cfg.d_model * cfg.mlp_hidden_size)
+        r["gemm_flops"] = tok * per_token + kept * 2 * cfg.d_model * cfg.vocab_size
+        r["query_tokens"] = tok
+    best = rows[-1] if len(rows) == 2 else max(rows[1:], key=lambda r: r["tokens_per_s"])
+    tflops = best["gemm_flops"] / best["seconds"] / 1e12
+    result = {
+        "metric": "engine generated tokens/s vs full affix recompute", "unit": "tokens/s", "value": best["tokens_per_s"],
+        "n_gpus": 1, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"configs[4]: LLaDA-8B shape ({cfg.n_layers} layers, d 4096, 32 heads, vocab 126464), random init, "
                                f"batch {args.engine_batch}, shared affix {args.engine_affix} ({args.engine_placement}) + 64-256 request tokens, "
                                f"gen_length {gen}, block_length 32, threshold 0.9 (random weights: ~1 token per step, worst-case NFE)"},
-        "results": rows}))
+        "full_recompute_tokens_per_s": base, "speedup_vs_full_recompute": best["speedup_vs_full_recompute"],
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel": "whole engine loop (library GEMMs at M = 512 dominate)",
+                     "note": f"matrix-product flops of all forwards of the {best['mode']} run (attention excluded) over its wall time"},
+        "results": rows}
+    if cpu_baseline:
+        result["cpu_baseline"] = cpu_engine_baseline(torch, cfg, rows)
+    return result
 
 
 def main():
@@ -427,6 +650,8 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="layers of the relocation workload (32 = LLaDA-8B)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-attention", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the configs[0] and configs[2] legs")
+    ap.add_argument("--no-engine", action="store_true", help="skip the configs[4] engine leg (about a minute)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run three plain 1 GiB device copies (known traffic, to scale rocprofv3's FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--attention-shapes", action="store_true", help="only run the attention kernel on a few uniform shapes")
@@ -472,7 +697,7 @@ def main():
         kernel_sweep(torch, device, ops, args.steps)
         return
     if args.engine:
-        engine_bench(torch, device, args)
+        print(json.dumps(engine_bench(torch, device, args)))
         return
 
     wl = build_relocation_workload(torch, device, args.layers)
@@ -532,6 +757,19 @@ def main():
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_relocation_baseline(torch, wl)
+    for name in list(wl):   # the 32-layer caches (18 GB): the legs below bring their own inputs
+        if torch.is_tensor(wl[name]):
+            del wl[name]
+    torch.cuda.empty_cache()
+
+    if not args.no_configs:
+        result["relocate_fp32"] = relocate_fp32_bench(torch, device, ops, max(args.steps, 20), args.warmup,
+                                                      cpu_baseline=not args.no_cpu_baseline)
+        result["anchor_select_scatter"] = anchor_select_scatter_bench(torch, device, ops, max(args.steps, 20), args.warmup,
+                                                                      cpu_baseline=not args.no_cpu_baseline)
+    if not args.no_engine:
+        result["engine"] = engine_bench(torch, device, args, ratios=[0.2], cpu_baseline=not args.no_cpu_baseline)
+    result["traffic_measured_at_commit"] = MEASURED_TRAFFIC_COMMIT
 
     print(json.dumps(result))
 

@@ -18,7 +18,11 @@ def test_more_than_one_gpu_is_refused():
 
 @pytest.mark.gpu
 def test_default_line_has_the_contract_keys(device):
-    proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--steps", "3", "--warmup", "1", "--layers", "4"],
+    # the relocation leg on 4 of 32 layers and the engine leg on a 2-layer model with 4 short requests: same code
+    # paths and keys as the default run, a fraction of its time
+    proc = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--steps", "3", "--warmup", "1", "--layers", "4",
+                           "--engine-layers", "2", "--engine-batch", "4", "--engine-gen", "32", "--engine-affix", "300",
+                           "--engine-kv-blocks", "24"],
                           capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stderr[-2000:]
     lines = [l for l in proc.stdout.splitlines() if l.strip()]
@@ -36,3 +40,12 @@ def test_default_line_has_the_contract_keys(device):
     a = d["attention"]
     assert a["roofline"]["bound"] == "mfma" and a["roofline"]["peak"] == 2500.0 and a["value"] > 0
     assert a["cpu_baseline"]["value"] > 0
+    for name, bound in (("relocate_fp32", "hbm"), ("anchor_select_scatter", "hbm"), ("engine", "mfma")):
+        leg = d[name]
+        assert "workload" in leg["config"] and leg["value"] > 0, name
+        assert leg["roofline"]["bound"] == bound and abs(leg["roofline"]["frac"] - leg["roofline"]["achieved"] / leg["roofline"]["peak"]) < 1e-3
+        assert leg["cpu_baseline"]["value"] > 0 and leg["cpu_baseline"]["sample"], name
+    assert d["relocate_fp32"]["affix_only"]["rows"] == 512 and d["relocate_fp32"]["whole_buffer"]["rows"] == 896
+    assert d["anchor_select_scatter"]["topk"]["us_per_launch"] > 0
+    modes = [r["mode"] for r in d["engine"]["results"]]
+    assert modes == ["full_recompute", "acache_0.2"] and d["engine"]["speedup_vs_full_recompute"] > 0

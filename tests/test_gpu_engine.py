@@ -68,7 +68,7 @@ def test_admission_out_of_memory_shrinks_the_cache_and_restores_it(device, capsy
         runner = ModelRunner(model, _serve(cfg, num_kvcache_blocks=12))
         seqs = requests()
         prefix = runner._prepare_acache(seqs)
-        real, sizes = runner._compute_anchor_positions_batch, []
+        real, sizes = runner._select_anchors_on_device, []
 
         def probe(batch):
             sizes.append(int(runner.config.num_kvcache_blocks))
@@ -76,7 +76,7 @@ def test_admission_out_of_memory_shrinks_the_cache_and_restores_it(device, capsy
                 raise torch.OutOfMemoryError("forced by the test")
             return real(batch)
 
-        runner._compute_anchor_positions_batch = probe
+        runner._select_anchors_on_device = probe
         with torch.inference_mode():
             runner._prepare_admitted_sequences_for_acache(seqs, prefix, allow_kv_cache_resize=allow)
         return runner, seqs, sizes
@@ -346,19 +346,62 @@ def test_batched_probe_at_admission_selects_the_same_anchors(device, placement, 
         runner = ModelRunner(model, _serve(cfg, recompute_batch_size=2, max_num_seqs=0, num_kvcache_blocks=40,
                                            anchor_ratio=0.4, anchor_selection_batch_size=probe_batch))
         calls = []
-        real = runner._compute_anchor_positions_batch
+        real = runner._select_anchors_on_device      # batched serving keeps the anchors on the device
 
         def spy(batch, real=real, calls=calls):
             calls.append(len(batch))
             return real(batch)
 
-        runner._compute_anchor_positions_batch = spy
+        runner._select_anchors_on_device = spy
         seqs = [make(i) for i in range(5)]
         out, _ = runner.generate_with_acache(seqs)
-        results.append(([list(s.anchor_positions) for s in seqs], out))
+        assert all(s.device_layout is not None for s in seqs)
+        results.append(([list(s.anchor_positions) for s in seqs], out))   # read back on demand
         assert calls == {1: [1] * 5, 0: [5], 3: [3, 2]}[probe_batch]
     assert results[0] == results[1] == results[2]
     assert all(len(a) == 5 for a in results[0][0])          # ceil(0.4 * 12) anchors per request
+
+
+def test_device_layouts_equal_the_host_layouts(device):
+    """Batched serving keeps anchors and slot maps on the device.  What the layout launch produced for the admitted
+    requests must be, list for list, what ``Sequence.finalize_slot_mapping`` builds on the host from the same
+    anchors and block tables, and the packed read order must be the host's query-relocation order."""
+    cfg, model = _model(device, seed=3)
+    affix = list(range(20, 32))
+
+    def make(i):
+        if i % 2:
+            return Sequence(affix + [40 + i, 41 + i], gen_length=4, block_length=4, cache_block_size=8, mask_id=63,
+                            prompt_affix_len=len(affix))
+        return Sequence([2 + i] * (1 + i) + affix + [40 + i], gen_length=4, block_length=4, cache_block_size=8,
+                        mask_id=63, prompt_affix_start=1 + i, prompt_affix_end=1 + i + len(affix))
+
+    runner = ModelRunner(model, _serve(cfg, max_num_seqs=0, num_kvcache_blocks=40, anchor_ratio=0.4))
+    seqs = [make(i) for i in range(4)]
+    with torch.inference_mode():
+        prefix = runner._prepare_acache(seqs)
+        batch = []
+        assert runner._admit_sequences_with_acache(batch, seqs, prefix, True) == 4
+    for seq in seqs:
+        layout = seq.device_layout
+        assert layout is not None and layout.anchors.dtype == torch.int32
+        twin = Sequence(seq.token_ids[: seq.num_prompt_tokens], gen_length=4, block_length=4, cache_block_size=8,
+                        mask_id=63, prompt_affix_start=seq.affix_start, prompt_affix_end=seq.affix_end)
+        twin.enable_acache(len(affix), 0.4, affix_start=seq.affix_start, affix_end=seq.affix_end)
+        twin.set_anchor_positions(layout.anchors.tolist())
+        twin.block_table = list(seq.block_table)
+        twin.finalize_slot_mapping()
+        assert seq.anchor_positions == twin.anchor_positions and len(twin.anchor_positions) == 5
+        assert seq.read_slot_map == twin.read_slot_map
+        assert seq.recompute_positions == twin.recompute_positions
+        assert seq.recompute_slot_mapping == twin.recompute_slot_mapping
+        assert seq.block_query_start() == twin.recompute_positions.index(twin.generation_start)
+        assert layout.tokens.tolist() == seq.token_ids
+        want, shared = runner._attention_read_layout(twin, True)
+        if seq.affix_start:
+            assert layout.read_packed.tolist() == want and shared == seq.affix_len - seq.num_anchor_tokens
+        else:
+            assert layout.read_packed is None and shared == 0
 
 
 def test_merged_projections_keep_the_state_dict_and_follow_parameter_updates(device):

@@ -51,7 +51,8 @@ def test_importance_matches_the_reference_fixture(device):
         assert got.shape == want.shape
         torch.testing.assert_close(got, want, rtol=8e-2, atol=1e-1, msg=lambda m: f"{c['name']}: {m}")
         k = G.ceil_to_int(kw["anchor_ratio"] * want.shape[1])
-        assert G.select_anchor_tokens(got, k, "top").tolist() == G.select_anchor_tokens(want, k, "top").tolist(), c["name"]
+        assert (G.select_anchor_tokens(got.to(device), k, "top").tolist()
+                == G.select_anchor_tokens(want.to(device), k, "top").tolist()), c["name"]
 
 
 @pytest.mark.parametrize("from_cache", [True, False])
