@@ -26,6 +26,7 @@
 
 #include "common.h"
 #include "mma.h"
+#include "attn_common.h"
 
 namespace acache {
 
@@ -310,6 +311,268 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The same two passes for head dims of 64, 128 and 256 with the streamed operand staged through LDS.
+// In the kernels above every wave pulls the streamed rows (keys in the statistics pass, queries in the
+// column pass) from L2 in operand layout, 64 bytes of a row per four lanes: the workgroup's four waves ask
+// for the same or neighbouring rows four times over and the vector memory path, not the matrix core, sets
+// the pace.  Here the four waves of a workgroup share one stream: the copy engine writes each 32-row tile
+// into LDS once (whole rows, 16 bytes per lane, two buffers in turn) and all four waves read their
+// fragments from there.  Rows are laid out with the 16-byte chunks of row r XOR-ed by r, so that the 16
+// lanes reading one chunk column of 16 different rows hit 16 different bank groups.
+constexpr int kStageRows = 32;  // query rows per LDS tile of the column pass
+constexpr int kStageKeys = 64;  // keys per LDS tile of the statistics pass
+
+template <int D, int ROWS>
+struct StageGeometry {
+  static constexpr int kChunks = D / 8;                   // 16-byte chunks per row (a power of two)
+  static constexpr int kTileBytes = ROWS * D * 2;
+  static constexpr int kCopiesPerWave = ROWS * D / 2048;  // 1 KiB wave copies per tile, split over four waves
+  // chunk `c` of tile row `row` lives at this byte offset of the tile
+  static __device__ __forceinline__ int offset(int row, int c) { return row * (D * 2) + ((c ^ (row & (kChunks - 1))) << 4); }
+};
+
+// Fragment of tile rows 16*t + li from LDS, in the layout load_rows() produces from global memory.
+template <int D>
+__device__ __forceinline__ void load_rows_lds(vec16 (&f)[D / 32], const char *tile, int t, int li, int lg) {
+  using G = StageGeometry<D, 16>;  // the offset of a chunk does not depend on the tile height
+#pragma unroll
+  for (int ks = 0; ks < D / 32; ++ks) f[ks] = *(const vec16 *)(tile + G::offset(16 * t + li, 4 * ks + lg));
+}
+
+// Make the compiler finish a register-resident fragment's loads here.  Left alone it waits where the fragment is
+// first used, inside the streaming loop, with a count that knows nothing of the LDS copies in flight there: a
+// wait for "everything I issued" then also drains the copy of the next tile, every step.
+__device__ __forceinline__ void settle(const vec16 &v) {
+  asm volatile("" ::"v"(v.w[0]), "v"(v.w[1]), "v"(v.w[2]), "v"(v.w[3]));
+}
+
+// One workgroup per (request, head, 256 mask rows): wave w keeps rows 64*w .. 64*w + 63 in registers, the
+// affix keys stream through LDS 32 at a time.  Same arithmetic and the same statistic as importance_stats_kernel.
+template <int DTYPE, int D>
+__global__ __launch_bounds__(256) void importance_stats_lds_kernel(ImportanceParams p) {
+  constexpr int NQ = kRowTilesPerWave, KS = D / 32, NT = 2;  // key tiles scored together (a 64-key LDS tile: two rounds)
+  using M = Mma<DTYPE>;
+  using G = StageGeometry<D, kStageKeys>;
+  __shared__ __attribute__((aligned(1024))) char tiles[2][G::kTileBytes];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 15, lg = lane >> 4;
+  const int groups = (p.max_row_tiles + 4 * NQ - 1) / (4 * NQ);
+  const int b = blockIdx.x / groups, rg = blockIdx.x % groups;
+  const int h = blockIdx.y;
+  const int m0 = p.cu_mask[b];
+  const int n_rows = p.cu_mask[b + 1] - m0;
+  if (rg * 4 * NQ * 16 >= n_rows) return;  // the whole workgroup: nothing to score
+  const int row0 = (rg * 4 + wave) * NQ * 16;
+  const bool live = row0 < n_rows;  // a wave past the request's rows still copies and synchronises
+  const int kvh = h / (p.H / p.H_kv);
+  const float c = p.scale_log2e;
+
+  vec16 qf[NQ][KS];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) load_rows<D>(qf[qt], mask_query_row(p, m0, n_rows, row0 + 16 * qt + li, h), lg);
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) settle(qf[qt][ks]);
+
+  // this lane's share of a tile copy: chunk slot `lane` of the 1 KiB piece (wave, j) holds which row and chunk?
+  const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
+  int copy_row[G::kCopiesPerWave], copy_off[G::kCopiesPerWave];
+#pragma unroll
+  for (int j = 0; j < G::kCopiesPerWave; ++j) {
+    const int slot = (wave * G::kCopiesPerWave + j) * 64 + lane;
+    copy_row[j] = slot / G::kChunks;
+    copy_off[j] = ((slot % G::kChunks) ^ (copy_row[j] & (G::kChunks - 1))) << 4;
+  }
+  auto issue = [&](int a0, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < G::kCopiesPerWave; ++j) {
+      const int a = a0 + copy_row[j];
+      lds_dma16(k_base + (int64_t)(a < p.A ? a : p.A - 1) * p.kv_slot_bytes + copy_off[j],
+                tiles[buf] + (wave * G::kCopiesPerWave + j) * 1024);
+    }
+  };
+
+  float m_run[NQ], l_run[NQ];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) { m_run[qt] = -INFINITY; l_run[qt] = 0.0f; }
+  issue(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int t0 = 0, it = 0; t0 < p.A; t0 += kStageKeys, ++it) {
+    issue(t0 + kStageKeys, (it + 1) & 1);  // always: past the end the last key is re-read and ignored
+    if (live) {
+      const char *tile = tiles[it & 1];
+#pragma unroll
+     for (int half = 0; half < kStageKeys / (16 * NT); ++half) {
+      const int a0 = t0 + 16 * NT * half;
+      if (a0 >= p.A) break;  // wave-uniform
+      const bool tail = a0 + 16 * NT > p.A;
+      vec16 kf[NT][KS];
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) load_rows_lds<D>(kf[nt], tile, NT * half + nt, li, lg);
+#pragma unroll
+      for (int qp = 0; qp < NQ; qp += 2) {
+        f32x4 sc[2][NT];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) sc[u][nt] = f32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) sc[u][nt] = M::run(kf[nt][ks], qf[qp + u][ks], sc[u][nt]);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int qt = qp + u;
+          if (tail) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (a0 + 16 * nt + 4 * lg + i >= p.A) sc[u][nt][i] = -INFINITY;
+          }
+          float mx = -INFINITY;
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sc[u][nt][i]);
+          mx = fmaxf(mx, __shfl_xor(mx, 16));
+          mx = fmaxf(mx, __shfl_xor(mx, 32));
+          const float m_new = fmaxf(m_run[qt], mx * c);
+          float add = 0.0f;
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(sc[u][nt][i] * c - m_new);
+          l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + add;
+          m_run[qt] = m_new;
+        }
+      }
+     }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next tile has landed ...
+    __syncthreads();                                    // ... and everybody is done with this one
+  }
+  if (!live) return;
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    float l = l_run[qt];
+    l += __shfl_xor(l, 16);
+    l += __shfl_xor(l, 32);
+    const int r = row0 + 16 * qt + li;
+    if (lg == 0 && r < n_rows) {
+      const int64_t src_row = p.mask_rows[m0 + r];
+      const bool present = src_row >= 0 && src_row < p.total_q;
+      p.stats[(int64_t)(m0 + r) * p.H + h] = present ? m_run[qt] + __builtin_amdgcn_logf(l) : INFINITY;
+    }
+  }
+}
+
+// One workgroup per (request, head, 256 affix keys): wave w keeps keys 64*w .. 64*w + 63 of the block in
+// registers, the request's mask rows stream through LDS 32 at a time.  Same arithmetic as importance_colsum_kernel.
+template <int DTYPE, int D>
+__global__ __launch_bounds__(256) void importance_colsum_lds_kernel(ImportanceParams p) {
+  constexpr int KS = D / 32, NR = kStageRows / 16;
+  using M = Mma<DTYPE>;
+  using G = StageGeometry<D, kStageRows>;
+  __shared__ __attribute__((aligned(1024))) char tiles[2][G::kTileBytes];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane & 15, lg = lane >> 4;
+  const int b = blockIdx.z;
+  const int h = blockIdx.y;
+  const int a0 = blockIdx.x * (4 * kKeysPerStep) + wave * kKeysPerStep;
+  const int m0 = p.cu_mask[b];
+  const int n_rows = p.cu_mask[b + 1] - m0;
+  const bool live = a0 < p.A;  // a wave past the affix still copies and synchronises
+  if (n_rows <= 0) {          // the whole workgroup: a request without mask rows has all-zero sums
+    float *zero = p.partial + ((int64_t)b * p.H + h) * p.A;
+    if (a0 + lane < p.A) zero[a0 + lane] = 0.0f;
+    return;
+  }
+  const float c = p.scale_log2e;
+  const int kvh = h / (p.H / p.H_kv);
+  const char *k_base = p.k_cache + p.affix_slot0 * p.kv_slot_bytes + (int64_t)kvh * p.kv_head_bytes;
+
+  vec16 kf[4][KS];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int a = a0 + 16 * nt + li;
+    load_rows<D>(kf[nt], k_base + (int64_t)(a < p.A ? a : p.A - 1) * p.kv_slot_bytes, lg);
+  }
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) settle(kf[nt][ks]);
+  int copy_row[G::kCopiesPerWave], copy_off[G::kCopiesPerWave];
+#pragma unroll
+  for (int j = 0; j < G::kCopiesPerWave; ++j) {
+    const int slot = (wave * G::kCopiesPerWave + j) * 64 + lane;
+    copy_row[j] = slot / G::kChunks;
+    copy_off[j] = ((slot % G::kChunks) ^ (copy_row[j] & (G::kChunks - 1))) << 4;
+  }
+  auto issue = [&](int r0, int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < G::kCopiesPerWave; ++j)
+      lds_dma16(mask_query_row(p, m0, n_rows, r0 + copy_row[j], h) + copy_off[j],
+                tiles[buf] + (wave * G::kCopiesPerWave + j) * 1024);
+  };
+  auto statistic = [&](int r0, float (&st)[NR]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int t = 0; t < NR; ++t) {
+      const int r = r0 + 16 * t + li;
+      st[t] = p.stats[(int64_t)(m0 + (r < n_rows ? r : n_rows - 1)) * p.H + h];
+    }
+  };
+  float col[4][4] = {};
+  float st_cur[NR], st_next[NR];
+  statistic(0, st_cur);
+  issue(0, 0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  for (int r0 = 0, it = 0; r0 < n_rows; r0 += kStageRows, ++it) {
+    statistic(r0 + kStageRows, st_next);       // ordinary loads first, then the copies behind them
+    issue(r0 + kStageRows, (it + 1) & 1);      // always: past the end the last row is re-read and ignored
+    if (live) {
+      const char *tile = tiles[it & 1];
+#pragma unroll
+      for (int t = 0; t < NR; ++t) {
+        const float ref = r0 + 16 * t + li < n_rows ? st_cur[t] : INFINITY;  // 2^-inf = 0 for rows past the end
+        vec16 qf[KS];
+        load_rows_lds<D>(qf, tile, t, li, lg);
+        f32x4 sc[4];
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) sc[nt] = f32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+          for (int nt = 0; nt < 4; ++nt) sc[nt] = M::run(kf[nt][ks], qf[ks], sc[nt]);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(sc[nt][i] * c - ref);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < NR; ++t) st_cur[t] = st_next[t];
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next tile has landed ...
+    __syncthreads();                                    // ... and everybody is done with this one
+  }
+  if (!live) return;
+  float *dst = p.partial + ((int64_t)b * p.H + h) * p.A;
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float v = row_sum16(col[nt][i]);
+      const int a = a0 + 16 * nt + 4 * lg + i;
+      if (li == 0 && a < p.A) dst[a] = v;
+    }
+}
+
 // importance[b, a] += sum over heads of partial[b, h, a], in a fixed order: four lanes take every fourth head
 // each (their loads all in flight together), then the four shares are added in lane order.
 __global__ __launch_bounds__(256) void importance_reduce_kernel(ImportanceParams p) {
@@ -410,17 +673,30 @@ static int importance_launch(
   const dim3 grid1((unsigned)((int64_t)B * row_groups), (unsigned)((H + 3) / 4));
   const dim3 grid2((unsigned)((affix_len + kKeysPerStep - 1) / kKeysPerStep), (unsigned)((H + 3) / 4), (unsigned)B);
   const dim3 grid3((unsigned)((affix_len + 63) / 64), (unsigned)B);
+  // the LDS-staged pair: a workgroup per (request, head, 256 mask rows) and per (request, head, 256 affix keys)
+  const int row_groups_staged = (p.max_row_tiles + 4 * kRowTilesPerWave - 1) / (4 * kRowTilesPerWave);
+  const dim3 grid1s((unsigned)((int64_t)B * row_groups_staged), (unsigned)H);
+  const dim3 grid2s((unsigned)((affix_len + 4 * kKeysPerStep - 1) / (4 * kKeysPerStep)), (unsigned)H, (unsigned)B);
 #define ACACHE_CASE(DT, HD)                                                                       \
   if (dtype == DT && D == HD) {                                                                   \
     hipLaunchKernelGGL((importance_rotate_kernel<DT>), grid0, dim3(256), 0, s, p);                \
     const int rc0 = launch_status("importance_rotate_kernel");                                    \
     if (rc0) return rc0;                                                                          \
-    hipLaunchKernelGGL((importance_stats_kernel<DT, HD>), grid1, dim3(256), 0, s, p);             \
-    const int rc = launch_status("importance_stats_kernel");                                      \
-    if (rc) return rc;                                                                            \
-    hipLaunchKernelGGL((importance_colsum_kernel<DT, HD>), grid2, dim3(256), 0, s, p);            \
-    const int rc2 = launch_status("importance_colsum_kernel");                                    \
-    if (rc2) return rc2;                                                                          \
+    if constexpr (HD == 64 || HD == 128 || HD == 256) {                                           \
+      hipLaunchKernelGGL((importance_stats_lds_kernel<DT, HD>), grid1s, dim3(256), 0, s, p);      \
+      const int rc = launch_status("importance_stats_lds_kernel");                                \
+      if (rc) return rc;                                                                          \
+      hipLaunchKernelGGL((importance_colsum_lds_kernel<DT, HD>), grid2s, dim3(256), 0, s, p);     \
+      const int rc2 = launch_status("importance_colsum_lds_kernel");                              \
+      if (rc2) return rc2;                                                                        \
+    } else {                                                                                      \
+      hipLaunchKernelGGL((importance_stats_kernel<DT, HD>), grid1, dim3(256), 0, s, p);           \
+      const int rc = launch_status("importance_stats_kernel");                                    \
+      if (rc) return rc;                                                                          \
+      hipLaunchKernelGGL((importance_colsum_kernel<DT, HD>), grid2, dim3(256), 0, s, p);          \
+      const int rc2 = launch_status("importance_colsum_kernel");                                  \
+      if (rc2) return rc2;                                                                        \
+    }                                                                                             \
     hipLaunchKernelGGL(importance_reduce_kernel, grid3, dim3(256), 0, s, p);                      \
     return launch_status("importance_reduce_kernel");                                             \
   }

@@ -33,9 +33,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 # WRITE_SIZE runs of this script (raw counters scaled by what they read for the 1 GiB copy of
 # --copy-calibration), taken at the commit named here; profiles/*.md hold the summaries and their commands.
 # A kernel changed after that commit makes its figure stale: re-run the counters and update both.
-MEASURED_TRAFFIC_COMMIT = "TRAFFIC_COMMIT_PLACEHOLDER"
-MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 18.029e9, "attention": 284.5e6, "relocate_fp32": None,
-                          "scatter_28_layers": None}
+MEASURED_TRAFFIC_COMMIT = "a0b9e38"
+MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 18.029e9, "attention": 285.0e6, "relocate_fp32": 1.879e9,
+                          "scatter_28_layers": 332.1e6}
 
 
 def _event_times_ms(fn, steps, torch):
@@ -306,9 +306,7 @@ def anchor_select_scatter_bench(torch, device, ops, steps, warmup, cpu_baseline=
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES["scatter_28_layers"],
                      "kernel": "scatter_kernel<bf16>", "avg_launch_ms": round(timed["scatter"], 5),
-                     "algorithmic_bytes": scatter_bytes,
-                     "note": "166 MB written over a 332 MB working set: smaller than the 256 MB last-level cache, so "
-                             "part of the traffic never reaches HBM"},
+                     "algorithmic_bytes": scatter_bytes},
     }
     if cpu_baseline:
         torch.set_num_threads(os.cpu_count() or 1)
@@ -475,9 +473,9 @@ def kernel_sweep(torch, device, ops, steps):
     ws = torch.empty(ops.affix_importance_workspace_bytes(B * M, B, H, H, D, A, True), dtype=torch.uint8, device=device)
     us = timed(lambda: ops.affix_importance(imp, qp, kp, rows_p, cu_p, A, M, None, sh_p, cos, sin, 0, ws))
     flops = 2 * 2 * B * M * A * H * D   # the scores are computed twice (row statistics, then column sums)
-    out.append({"kernel": "importance kernels (rotate, stats, colsum, reduce)", "us": round(us, 1),
+    out.append({"kernel": "importance kernels (pack + counter-rotate queries, stats, colsum, reduce)", "us": round(us, 1),
                 "TFLOPs": round(flops / us / 1e6, 1), "flops": flops,
-                "workload": "one layer: 16 requests x 256 mask queries x 1 000 affix keys, 32 heads x 128, bf16, key-side re-rotation"})
+                "workload": "one layer: 16 requests x 256 mask queries x 1 000 affix keys, 32 heads x 128, bf16, relocated (shifts 1-255)"})
     logits = torch.randn(512, 126464, generator=gen, device=device).to(torch.bfloat16)
     row("confidence_kernel", timed(lambda: ops.argmax_confidence(logits)), 512 * 126464 * 2,
         "512 rows x 126 464 logits, bf16")
