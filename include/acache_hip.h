@@ -268,8 +268,12 @@ int acache_topk_anchors(
  * (nano-vdllm/model_runner.py:2279-2296: up-cast to fp32, gather of the chosen
  * logit, torch.logsumexp, exp) and the arg-max in front of it at temperature 0;
  * with temperature > 0 the caller draws the Gumbel arg-max itself and passes it
- * as `picks` (out_token may then be NULL).  The row is read once.  Logits are
- * assumed free of NaN.  row_stride in elements, a multiple of 16 bytes.
+ * as `picks` (out_token may then be NULL).  The row is read once.
+ * NaN: a NaN logit is never chosen as the arg-max (torch.argmax would return its
+ * index) but it enters the sum, so the row's confidence is NaN and the caller's
+ * `confidence >= threshold` test fails for it: on a row that holds a NaN this
+ * entry point and the reference's torch formulation may name different tokens, and
+ * neither commits one by threshold.  row_stride in elements, a multiple of 16 bytes.
  */
 int acache_argmax_confidence(
     int64_t *out_token, float *out_conf, const void *logits, const int64_t *picks,
@@ -348,17 +352,23 @@ int acache_build_slot_layout(
  * q / out: [total_q, H, D] with given token and head strides (innermost 1).
  * k_cache / v_cache: [num_slots, H_kv, D] with given slot and head strides.
  *
- * Schedule and workspace (head_dim 64 / 128, plain and query-side modes).  The kernel is launched as
- * a persistent grid of two workgroups per CU; the (request, 128-row query tile, head) units are laid
- * end to end and every workgroup takes an equal share of key-tile steps, so a unit may be cut between
- * neighbouring workgroups.  The parts of a cut unit meet in `workspace`: device memory of at least
+ * Schedule (head_dim 64 / 128).  One workgroup of four waves per (request, 128-row query tile, head)
+ * unit, two workgroups per CU, units handed out longest request first; K/V tiles of 64 keys reach LDS
+ * through the copy engine.  In key-side mode the rows of a tile that lie in shared slots are re-rotated
+ * in LDS after they land.  This schedule needs no workspace: pass NULL and 0.
+ *
+ * workspace / workspace_bytes are read only by an alternative schedule that the library takes when the
+ * environment holds ACACHE_ATTN_WIDE=1 (read once per process): eight waves per workgroup on 256-row
+ * units, one persistent workgroup per CU, the units laid end to end and cut into equal stretches of
+ * key-tile steps.  The parts of a cut unit meet in `workspace`: device memory of at least
  * acache_varlen_attn_workspace_bytes() bytes (a function of the current device's CU count: arrival
  * counters followed by two partial-state slots per workgroup), 16-byte aligned, owned by the caller.
  * Its counters must be ZERO before the first call that uses it (clear the buffer once after
- * allocating it); every call leaves them zero again, so the buffer is reusable as is.  Calls that
- * may overlap in time (different streams) need different workspaces.  The merge order is fixed, so
- * results are bit-identical from run to run.  workspace == NULL (or smaller than required): units are
- * never cut and are dealt whole instead — same results up to the rounding of the merge, longer tail.
+ * allocating it); every call leaves them zero again.  Calls that may overlap in time (different
+ * streams) need different workspaces.  The merge order is fixed, so results are bit-identical from
+ * run to run; against the default schedule they differ by the rounding of the merge.  With
+ * workspace == NULL (or too small) that schedule deals units whole.  It is faster on uniform
+ * batches of long requests and slower on ragged ones, which is why it is not the default.
  */
 int64_t acache_varlen_attn_workspace_bytes(void);
 int acache_varlen_attn(
