@@ -384,7 +384,8 @@ __global__ __launch_bounds__(256, RAGGED ? 1 : 2) void varlen_attn_kernel(AttnPa
 // 4*j + i/4, j = 0..3.  With lane l pointing at V[row0 + l/4][d0 + 4*(l%4)] lane i
 // gets V[row0 + 0..3][d0 + i]: four keys of one column, i.e. half of an MFMA
 // A-operand of V^T.
-// One query tile of one (request, head): the NW waves take WQ = 16 * NQ16 query rows each, starting at row
+// One query tile of one (request, head): the NW waves (4 in every instantiation; the tile geometry below is
+// written in terms of NW so that it stays in one place) take WQ = 16 * NQ16 query rows each, starting at row
 // q_tile0 of the request, and stream the request's key tiles [t_begin, t_end) through the LDS ring.
 template <int DTYPE, int D, int NQ16, int MODE, int NW = 4>
 __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0, char *lds_v0, char *lds_k1,
@@ -406,8 +407,9 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   constexpr int TILE_BYTES = BN * ROW_BYTES;
   using M = Mma<DTYPE>;
   typedef short s16x4 __attribute__((ext_vector_type(4)));
-  // An opaque zero ties the lane-derived address constants below to this call: otherwise the compiler hoists them
-  // out of the persistent loop around it and spills them to keep them alive across units.
+  // An opaque zero ties the lane-derived address constants below to this call: a caller that walks several parts
+  // in a loop would otherwise see them hoisted out of its loop and spilled to stay alive across parts.  With one
+  // part per workgroup, as the unit kernel calls it, it costs one scalar move.
   int opaque_zero;
   asm volatile("s_mov_b32 %0, 0" : "=s"(opaque_zero));
   const int tid = threadIdx.x + opaque_zero;
