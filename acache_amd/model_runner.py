@@ -917,6 +917,13 @@ class ModelRunner:
         self._active_timing = timing
         total_start = self._start_timing()
 
+        # positions index the model's rotary table; the kernels clamp an out-of-table row for memory safety only
+        # (it would come back unrotated), so the length is checked here, on the host, where it is known
+        table_rows = getattr(cfg.hf_config, "max_sequence_length", None) or getattr(cfg.hf_config, "max_position_embeddings", None)
+        longest = max((len(seq) for seq in prompts), default=0)
+        if table_rows is not None and longest > int(table_rows):
+            raise ValueError(f"a request of {longest} tokens exceeds the model's rotary table of {int(table_rows)} positions")
+
         total_nfe = 0
         results = [None] * len(prompts)
         index_of = {seq.seq_id: i for i, seq in enumerate(prompts)}

@@ -197,3 +197,15 @@ def test_out_of_memory_at_admission_shrinks_retries_and_restores(capsys):
     with pytest.raises(torch.OutOfMemoryError):
         runner._prepare_admitted_sequences_for_acache(seqs, prefix, allow_kv_cache_resize=False)
     assert runner.kv_cache.shape[2] == 12
+
+
+def test_requests_longer_than_the_rotary_table_are_refused():
+    """Positions past the model's rotary table would be left unrotated by the kernels (they only clamp for memory
+    safety); the engine refuses such a request on the host before any forward."""
+    runner = _tiny_runner(num_kvcache_blocks=16, enable_acache=False)
+    runner.allocate_kv_cache(16)
+    runner.model = _StubForward(lambda tokens: torch.full_like(tokens, 7))
+    too_long = Sequence(list(range(2, 62)), gen_length=8, cache_block_size=8, block_length=4, mask_id=63)  # 68 > 64
+    with pytest.raises(ValueError, match="rotary table"):
+        runner.generate_with_dual_cache([too_long])
+    assert runner.model.calls == 0
