@@ -54,11 +54,12 @@ __global__ __launch_bounds__(kConfThreads) void confidence_kernel(ConfidencePara
   RowStat st{-INFINITY, 0.0f, INT64_MAX};
   auto take = [&](const float (&x)[VEC], int n, int64_t base) {
     float cm = -INFINITY;
-    int ci = 0;
-    for (int j = 0; j < n; ++j)
-      if (x[j] > cm) { cm = x[j]; ci = j; }  // strict: the first maximum wins
+    for (int j = 0; j < n; ++j) cm = fmaxf(cm, x[j]);  // NaN never wins: fmaxf returns the other operand
     if (cm == -INFINITY) return;             // nothing finite here: contributes zero
-    if (cm > st.m) {
+    if (cm > st.m) {                         // rare after the first chunks: only then look for the position
+      int ci = 0;
+      for (int j = n - 1; j >= 0; --j)
+        if (x[j] == cm) ci = j;              // the first maximum wins
       st.s *= __expf(st.m - cm);             // exp(-inf) = 0 on the first chunk
       st.m = cm;
       st.idx = base + ci;
@@ -70,12 +71,13 @@ __global__ __launch_bounds__(kConfThreads) void confidence_kernel(ConfidencePara
 
   const int64_t full = p.V / VEC;
   int64_t c = tid;
-  for (; c + 3 * kConfThreads < full; c += 4 * kConfThreads) {  // four independent loads before any use
-    vec16 raw[4];
+  constexpr int kInFlight = 4;  // independent loads before any use (8 measured no better)
+  for (; c + (kInFlight - 1) * kConfThreads < full; c += kInFlight * kConfThreads) {
+    vec16 raw[kInFlight];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) raw[u] = load16_stream(row + (c + u * kConfThreads) * 16);
+    for (int u = 0; u < kInFlight; ++u) raw[u] = load16_stream(row + (c + u * kConfThreads) * 16);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < kInFlight; ++u) {
       float x[VEC];
       E::unpack(raw[u], x);
       take(x, VEC, (c + u * kConfThreads) * VEC);
