@@ -510,12 +510,12 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     for (int i = 0; i < NI; ++i) in_range &= (uint32_t)slots[i] < slot_limit;
     return tr.n0 + BN <= tr.n_end && __builtin_amdgcn_ballot_w64(!in_range) == 0;
   };
+  // this wave's rows inside a tile as a scalar byte offset (the lane's data lands 16 * lane behind the destination)
+  const uint32_t wave_dst = __builtin_amdgcn_readfirstlane((uint32_t)(wave * WAVE_ROWS * ROW_BYTES));
   auto issue_rows = [&](int i, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
     const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
-    char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;  // wave-uniform; lane data lands at + lane*16
-    char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
-    lds_dma16(k_lane_src[i] + row_off, kdst);
-    lds_dma16(v_lane_src[i] + row_off, vdst);
+    lds_dma16_at(k_lane_src[i] + row_off, lds_offset_of(kbuf) + wave_dst + i * RPI * ROW_BYTES);
+    lds_dma16_at(v_lane_src[i] + row_off, lds_offset_of(vbuf) + wave_dst + i * RPI * ROW_BYTES);
   };
   auto issue_slow = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
     const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
@@ -525,12 +525,10 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
       const int r = dma_row0 + i * RPI;
       const bool present = tr.n0 + r < tr.n_end && (uint32_t)slots[i] < slot_limit;
       const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
-      char *kdst = kbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
-      char *vdst = vbuf + (wave * WAVE_ROWS + i * RPI) * ROW_BYTES;
       const char *ksrc = present ? k_lane_src[i] + row_off : zero;
       const char *vsrc = present ? v_lane_src[i] + row_off : zero;
-      lds_dma16(ksrc, kdst);
-      lds_dma16(vsrc, vdst);
+      lds_dma16_at(ksrc, lds_offset_of(kbuf) + wave_dst + i * RPI * ROW_BYTES);
+      lds_dma16_at(vsrc, lds_offset_of(vbuf) + wave_dst + i * RPI * ROW_BYTES);
     }
   };
   auto issue = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {

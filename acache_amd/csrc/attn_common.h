@@ -178,6 +178,17 @@ __device__ __forceinline__ void lds_dma16(const char *src, char *lds_dst) {
   asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "{m0}"(base) : "memory");
 }
 
+// The same copy with the destination given as a byte offset inside LDS.  Callers compute it from scalar values
+// (the ring buffer's offset, a constant once the buffer pointer is cast BEFORE any lane-derived term is added,
+// plus a wave offset taken through readfirstlane once), so the destination costs scalar adds: no 64-bit pointer
+// per copy in vector registers, no null check of a generic pointer, no readfirstlane pair per copy.
+__device__ __forceinline__ uint32_t lds_offset_of(const char *lds_ptr) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char *)lds_ptr;
+}
+__device__ __forceinline__ void lds_dma16_at(const char *src, uint32_t lds_offset) {
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "{m0}"(lds_offset) : "memory");
+}
+
 // Online-softmax update of one key tile, in two steps shared by both attention kernels so that
 // they round identically (key-side relocation must reproduce a materialised copy bit for bit).
 //
