@@ -33,8 +33,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 # WRITE_SIZE runs of this script (raw counters scaled by what they read for the 1 GiB copy of
 # --copy-calibration), taken at the commit named here; profiles/*.md hold the summaries and their commands.
 # A kernel changed after that commit makes its figure stale: re-run the counters and update both.
-MEASURED_TRAFFIC_COMMIT = "a0b9e38"
-MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 18.029e9, "attention": 285.0e6, "relocate_fp32": 1.879e9,
+MEASURED_TRAFFIC_COMMIT = "e7d225a"
+MEASURED_TRAFFIC_BYTES = {"relocate_32_layers": 18.029e9, "attention": 286.0e6, "relocate_fp32": 1.879e9,
                           "scatter_28_layers": 332.1e6}
 
 
