@@ -676,19 +676,21 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     if (n < kv_len && slot >= 0 && slot < p.shared_prefix_len && delta != 0 && ad < p.rope_rows) {
       char *row = kbuf + rot_row * ROW_BYTES;
       const int f = (rot_row / RW) % CH;
-      auto rotate_with = [&](const float *cr, const float *sr) __attribute__((always_inline)) {
+      auto rotate_with = [&](const float *cr, const float *sr, float sign) __attribute__((always_inline)) {
 #pragma unroll
         for (int k = 0; k < PER_THREAD; ++k) {
           const int c = (tid % (PAIRS / PER_THREAD)) * PER_THREAD + k;
           char *lo_p = row + ((c ^ f) << 4), *hi_p = row + (((c + PAIRS) ^ f) << 4);
           vec16 lo = load16(lo_p), hi = load16(hi_p);
-          rotate_pair_half_fast<DTYPE>(lo, hi, cr, sr, c * 8, D / 2, delta < 0 ? -1.0f : 1.0f);
+          rotate_pair_half_fast<DTYPE>(lo, hi, cr, sr, c * 8, D / 2, sign);
           store16(lo_p, lo);
           store16(hi_p, hi);
         }
       };
-      if (delta == shift0) rotate_with(lds_rope, lds_rope + D);  // separate calls: LDS reads here, global loads there
-      else rotate_with(p.cos_tab + (int64_t)ad * D, p.sin_tab + (int64_t)ad * D);
+      // separate calls: LDS reads here, global loads there.  The cached rows belong to shift0 >= 0, so their sign
+      // is the literal +1 and the multiplications by it fold away.
+      if (delta == shift0) rotate_with(lds_rope, lds_rope + D, 1.0f);
+      else rotate_with(p.cos_tab + (int64_t)ad * D, p.sin_tab + (int64_t)ad * D, delta < 0 ? -1.0f : 1.0f);
     }
     __syncthreads();  // the rotated rows are in place for everybody
   };
