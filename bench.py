@@ -73,12 +73,13 @@ def build_relocation_workload(torch, device, layers):
 
 
 def cpu_relocation_baseline(torch, wl, budget_s=20.0):
-    """Reference-style torch CPU path (index_select + x*cos + rot_half(x)*sin) on ONE layer of the workload."""
+    """Reference-style torch CPU path (index_select + x*cos + rot_half(x)*sin) on a quarter of the workload's layers."""
     from oracle import acache_oracle as O
 
     torch.set_num_threads(os.cpu_count() or 1)
-    k1 = wl["k"][0:1].cpu()
-    v1 = wl["v"][0:1].cpu()
+    n_layers = min(8, wl["layers"])
+    k1 = wl["k"][0:n_layers].cpu()
+    v1 = wl["v"][0:n_layers].cpu()
     slot, delta = wl["slot"].cpu(), wl["delta"].cpu()
     cos, sin = wl["cos"].cpu(), wl["sin"].cpu()
     times = []
@@ -92,22 +93,22 @@ def cpu_relocation_baseline(torch, wl, budget_s=20.0):
         if time.perf_counter() - t_begin > budget_s and len(times) >= 1:
             break
     med = statistics.median(times)
-    bytes_layer = 2 * 2 * wl["T"] * wl["H"] * wl["D"] * 2
-    return dict(value=bytes_layer / med / 1e9, unit="GB/s", cores=torch.get_num_threads(), kind="port",
-                sample=f"1 of {wl['layers']} layers of the same batch ({wl['T']} rows), median of {len(times)} runs after 2 warm-ups, {med * 1e3:.0f} ms each")
+    bytes_sample = n_layers * 2 * 2 * wl["T"] * wl["H"] * wl["D"] * 2
+    return dict(value=round(bytes_sample / med / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"{n_layers} of {wl['layers']} layers of the same batch ({wl['T']} rows), median of {len(times)} runs after 2 warm-ups, {med * 1e3:.0f} ms each")
 
 
 def cpu_attention_baseline(torch, q, kc, vc, w, budget_s=15.0):
     """Reference-style torch CPU path for the attention call: per request, gather K/V through the slot map and run
     ``F.scaled_dot_product_attention`` over all heads (the formulation of nano-vdllm/model_runner.py:385-399), bf16
-    inputs up-cast to fp32.  Timed on a bounded sample of the 16 requests."""
+    inputs up-cast to fp32.  Timed on the whole call (all requests, all heads)."""
     import torch.nn.functional as F
 
     torch.set_num_threads(os.cpu_count() or 1)
     H, D = q.shape[1], q.shape[2]
     qc, kf, vf = q.cpu(), kc.cpu().view(-1, kc.shape[-2], D), vc.cpu().view(-1, vc.shape[-2], D)
     cu_q, cu_k, slots = w["cu_q"].tolist(), w["cu_k"].tolist(), w["slot_map"].long()
-    sample = list(range(min(4, len(w["q_lens"]))))
+    sample = list(range(len(w["q_lens"])))
 
     def run():
         for b in sample:
