@@ -11,16 +11,17 @@
 // and the cached affix keys as they lie in the cache: one copy of the keys, shared by all requests and resident
 // in L2, instead of one re-rotated copy per request.  Three more launches, no atomics, so the result does not
 // depend on scheduling:
-//   1. importance_stats_kernel: one wave per (request, head, 64 mask rows) walks the affix keys and
-//      leaves log2 of the row's sum of 2^(score * c) in the workspace;
-//   2. importance_colsum_kernel: one wave per (request, head, 64 affix keys) keeps its keys in
-//      registers, walks the request's mask rows, recomputes the scores, normalises them with the
-//      stored row statistic (one subtraction in the exponent) and sums the columns; it is the only writer of its 64 entries of the
-//      per-head partial sums in the workspace;
+//   1. statistics pass: the mask rows of a wave stay in registers, the affix keys stream by, and the wave
+//      leaves log2 of each row's sum of 2^(score * c) in the workspace;
+//   2. column pass: the affix keys of a wave stay in registers, the request's mask rows stream by, the scores
+//      are recomputed, normalised with the stored row statistic (one subtraction in the exponent) and summed
+//      per key; each wave is the only writer of its entries of the per-head partial sums in the workspace;
 //   3. importance_reduce_kernel adds the per-head partial sums, in head order, to importance[b, :].
-// Scores come from the matrix core (S^T = K Q^T, keys as rows, one query column per lane).  K and Q
-// fragments are loaded straight from global memory in operand layout (16 bytes per lane); nothing goes
-// through LDS and there is no barrier.
+// Scores come from the matrix core (S^T = K Q^T, keys as rows, one query column per lane).  Both passes exist
+// twice: for head dims of 64, 128 and 256 the streamed operand is staged through LDS by the copy engine and
+// shared by the four waves of a workgroup (importance_*_lds_kernel, further down); every other head dim loads
+// its fragments straight from global memory in operand layout, 16 bytes per lane, without LDS or barriers
+// (importance_stats_kernel, importance_colsum_kernel).
 #include <mutex>
 #include <type_traits>
 
@@ -55,7 +56,22 @@ struct ImportanceParams {
   int32_t rope_rows;
   int32_t max_row_tiles;
   int32_t D;  // head_dim
+  int32_t total_mask_rows;  // entries of mask_rows, rows of the packed query copy and of stats
+  int32_t max_mask_rows;    // the launch grids cover this many mask rows per request
 };
+
+// First mask row and number of mask rows of request b, held to what the workspace and the launch grids were
+// sized for: the prefix sums live in device memory, where the host cannot check them, and a request that
+// claims more rows than the caller declared is cut there instead of being read past the buffers.
+__device__ __forceinline__ void request_rows(const ImportanceParams &p, int b, int &m0, int &n_rows) {
+  m0 = p.cu_mask[b];
+  m0 = m0 < 0 ? 0 : (m0 > p.total_mask_rows ? p.total_mask_rows : m0);
+  int n = p.cu_mask[b + 1] - m0;
+  const int room = p.total_mask_rows - m0;
+  n = n > room ? room : n;
+  n = n > p.max_mask_rows ? p.max_mask_rows : n;
+  n_rows = n < 0 ? 0 : n;
+}
 
 // Operand fragments of 16 rows x D, KS = ceil(D / 32) slabs of 32 elements: lane (li, lg) takes elements
 // 32*ks + 8*lg .. + 8 of row `row_ptr` (always a readable row: callers clamp indices instead of branching, so
@@ -84,8 +100,8 @@ __global__ __launch_bounds__(256) void importance_rotate_kernel(ImportanceParams
   const int half_bytes = D;  // D / 2 elements of 2 bytes
   const int lpr = half_bytes / 16;
   const int b = blockIdx.y;
-  const int m0 = p.cu_mask[b];
-  const int n_rows = p.cu_mask[b + 1] - m0;
+  int m0, n_rows;
+  request_rows(p, b, m0, n_rows);
   const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t row = g / lpr;
   const int lane = (int)(g - row * lpr);
@@ -143,8 +159,8 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
   const int groups = (p.max_row_tiles + NQ - 1) / NQ;
   const int b = blockIdx.x / groups, rg = blockIdx.x % groups;
   const int h = blockIdx.y * 4 + wave;
-  const int m0 = p.cu_mask[b];
-  const int n_rows = p.cu_mask[b + 1] - m0;
+  int m0, n_rows;
+  request_rows(p, b, m0, n_rows);
   const int row0 = rg * NQ * 16;
   if (h >= p.H || row0 >= n_rows) return;  // no barrier in this kernel: waves may leave early
   const int kvh = h / (p.H / p.H_kv);
@@ -247,8 +263,8 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
   const int b = blockIdx.z;
   const int h = blockIdx.y * 4 + wave;
   const int a0 = blockIdx.x * kKeysPerStep;
-  const int m0 = p.cu_mask[b];
-  const int n_rows = p.cu_mask[b + 1] - m0;
+  int m0, n_rows;
+  request_rows(p, b, m0, n_rows);
   if (h >= p.H) return;
   const float c = p.scale_log2e;
   const int kvh = h / (p.H / p.H_kv);
@@ -360,8 +376,8 @@ __global__ __launch_bounds__(256) void importance_stats_lds_kernel(ImportancePar
   const int groups = (p.max_row_tiles + 4 * NQ - 1) / (4 * NQ);
   const int b = blockIdx.x / groups, rg = blockIdx.x % groups;
   const int h = blockIdx.y;
-  const int m0 = p.cu_mask[b];
-  const int n_rows = p.cu_mask[b + 1] - m0;
+  int m0, n_rows;
+  request_rows(p, b, m0, n_rows);
   if (rg * 4 * NQ * 16 >= n_rows) return;  // the whole workgroup: nothing to score
   const int row0 = (rg * 4 + wave) * NQ * 16;
   const bool live = row0 < n_rows;  // a wave past the request's rows still copies and synchronises
@@ -485,8 +501,8 @@ __global__ __launch_bounds__(256) void importance_colsum_lds_kernel(ImportancePa
   const int b = blockIdx.z;
   const int h = blockIdx.y;
   const int a0 = blockIdx.x * (4 * kKeysPerStep) + wave * kKeysPerStep;
-  const int m0 = p.cu_mask[b];
-  const int n_rows = p.cu_mask[b + 1] - m0;
+  int m0, n_rows;
+  request_rows(p, b, m0, n_rows);
   const bool live = a0 < p.A;  // a wave past the affix still copies and synchronises
   if (n_rows <= 0) {          // the whole workgroup: a request without mask rows has all-zero sums
     float *zero = p.partial + ((int64_t)b * p.H + h) * p.A;
@@ -666,6 +682,8 @@ static int importance_launch(
   p.scale_log2e = scale * 1.4426950408889634f;
   p.A = affix_len; p.B = B; p.H = H; p.H_kv = H_kv; p.rope_rows = rope_rows; p.D = D;
   p.max_row_tiles = (max_mask_rows + 15) / 16;
+  p.total_mask_rows = (int32_t)total_mask_rows;
+  p.max_mask_rows = max_mask_rows;
   hipStream_t s = (hipStream_t)stream;
   const int lanes_per_row = D * 2 / 32;
   const dim3 grid0((unsigned)(((int64_t)max_mask_rows * H * lanes_per_row + 255) / 256), (unsigned)B);

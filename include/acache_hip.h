@@ -190,9 +190,11 @@ int acache_rope_qk_scatter(
  * [0, total_q) is an absent query and adds nothing.  workspace:
  * device scratch of at least acache_affix_importance_workspace_bytes(total_mask_rows, B, H,
  * H_kv, D, affix_len, relocated = affix_shifts != NULL) bytes (row statistics, per-head
- * partial sums and, with relocation, the counter-rotated copy of the mask queries,
+ * partial sums and the packed, counter-rotated copy of the mask queries,
  * passed between the launches), 16-byte aligned, owned by the caller.  max_mask_rows: an upper bound on
- * the mask rows of one request.  D: a multiple of 16 up to 256; dtype bf16 or f16.
+ * the mask rows of one request; a request whose cu_mask entries claim more rows than that, or more than
+ * total_mask_rows leaves room for, is scored on the rows that fit (cu_mask is device memory the host does
+ * not read).  D: a multiple of 16 up to 256; dtype bf16 or f16.
  */
 int64_t acache_affix_importance_workspace_bytes(int64_t total_mask_rows, int32_t B, int32_t H, int32_t H_kv,
                                                 int32_t D, int32_t affix_len, int32_t relocated);
@@ -351,6 +353,9 @@ int acache_build_slot_layout(
  * slot lies outside [0, num_slots) reads as a zero row.
  * q / out: [total_q, H, D] with given token and head strides (innermost 1).
  * k_cache / v_cache: [num_slots, H_kv, D] with given slot and head strides.
+ * cu_q / cu_k are device memory and taken as given, as the reference takes its cu_seqlens:
+ * non-decreasing prefix sums of B + 1 entries with cu_q[0] == cu_k[0] == 0, cu_q[B] == total_q and
+ * cu_k[B] == total_k (the length of slot_map).  Slot values are checked per key, the prefix sums are not.
  *
  * Schedule (head_dim 64 / 128).  One workgroup of four waves per (request, 128-row query tile, head)
  * unit, two workgroups per CU, units handed out longest request first; K/V tiles of 64 keys reach LDS

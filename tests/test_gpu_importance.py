@@ -68,6 +68,26 @@ def test_mask_rows_outside_q_are_absent_queries(device):
         assert torch.allclose(got, clean, rtol=1e-5, atol=1e-6)   # same rows, another tiling of them
 
 
+def test_row_counts_beyond_the_declared_sizes_are_cut(device):
+    """The prefix sums are device memory the host cannot check: a request that claims more mask rows than the
+    index tensor holds, or than `max_mask_rows` says, is cut to what was declared."""
+    _, _, (q, kc, rows, cu, args) = _case(device, 8, 2, 128, A=90, mask_counts=[20, 6], shifts=[9, 2], seed=12)
+    clean = torch.zeros(2, 90, dtype=torch.float32, device=device)
+    ops.affix_importance(clean, q.to(device), kc.to(device), rows.to(device), cu.to(device), 90, 20, **args)
+    got = torch.zeros_like(clean)
+    claims_too_many = torch.tensor([0, 20, 40], dtype=torch.int32, device=device)   # 26 rows exist
+    ops.affix_importance(got, q.to(device), kc.to(device), rows.to(device), claims_too_many, 90, 20, **args)
+    assert torch.equal(got, clean)
+    # max_mask_rows = 6: the first request is scored on its first 6 rows only, the second is unchanged
+    short = torch.zeros_like(clean)
+    ops.affix_importance(short, q.to(device), kc.to(device), rows.to(device), cu.to(device), 90, 6, **args)
+    first6 = torch.zeros_like(clean)
+    cu6 = torch.tensor([0, 6, 6], dtype=torch.int32, device=device)
+    ops.affix_importance(first6, q.to(device), kc.to(device), rows.to(device), cu6, 90, 6, **args)
+    assert torch.equal(short[1], clean[1])
+    assert torch.allclose(short[0], first6[0], rtol=1e-6, atol=1e-7)
+
+
 def test_argument_errors(device):
     q = torch.zeros(4, 2, 128, dtype=torch.bfloat16, device=device)
     kc = torch.zeros(8, 2, 128, dtype=torch.bfloat16, device=device)
