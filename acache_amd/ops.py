@@ -376,8 +376,9 @@ def affix_importance(
 
 def affix_importance_workspace_bytes(total_mask_rows: int, batch: int, num_heads: int, num_kv_heads: int,
                                      head_dim: int, affix_len: int, relocated: bool) -> int:
-    """Bytes of scratch ``affix_importance`` needs: row statistics, per-head partial sums and, when
-    ``affix_shifts`` are given, the counter-rotated copy of the [MASK] queries."""
+    """Bytes of scratch ``affix_importance`` needs: row statistics, per-head partial sums and the packed copy of
+    the [MASK] queries (counter-rotated when ``affix_shifts`` are given; made either way, so ``relocated`` does
+    not change the size)."""
     return int(_lib.load().acache_affix_importance_workspace_bytes(
         total_mask_rows, batch, num_heads, num_kv_heads, head_dim, affix_len, int(relocated)))
 
