@@ -10,7 +10,10 @@ algorithm — affix K/V computed once, K anchors chosen by cross-affix importanc
 non-affix tokens recomputed at every block boundary, block-only refinement in between — runs on
 the paged engine of this package (``ModelRunner`` + HIP kernels).  Consequences for callers:
 
-* ``model`` is an engine model (``acache_amd.llada.LLaDAModelLM``) or a ready ``ModelRunner``;
+* ``model`` is the checkpoint model object the reference's caller passes (llada/eval_ACache.py:100-107, 189):
+  the engine model is built around its parameter tensors on first use (no second copy of the weights; settings
+  the engine's decoder stack does not implement raise ``TypeError``).  An engine model
+  (``acache_amd.llada.LLaDAModelLM``) or a ready ``ModelRunner`` is taken as it is;
 * ``precomputed_affix_cache`` is optional.  ``None``: the affix is encoded once into the shared
   slots.  A per-layer tuple of ``(k, v)`` with the HF layout ``[1, H_kv, A, D]`` and PRE-RoPE keys
   (llada/generate_ACache.py:153) is rotated to positions ``0..A-1`` and scattered into the shared
@@ -21,6 +24,7 @@ the paged engine of this package (``ModelRunner`` + HIP kernels).  Consequences 
 """
 from __future__ import annotations
 
+import weakref
 from typing import Optional, Tuple
 
 import torch
@@ -136,6 +140,42 @@ def get_transfer_index_dynamic(logits, temperature, remasking, mask_index, x, nu
 
 
 # ------------------------------------------------------------------------------------------ engine glue
+_ADOPTED = weakref.WeakKeyDictionary()   # checkpoint model object -> the engine model built around its weights
+
+
+def _engine_model(model):
+    """``model`` itself when it is one of this package's models; for the checkpoint model object the HF path
+    passes (llada/eval_ACache.py:100-107, 189; dream/eval_ACache.py likewise), the engine model built around the
+    same parameter tensors, made once per object."""
+    inner = getattr(model, "model", None)
+    if (inner is not None and hasattr(model, "config")
+            and any(hasattr(m, "k_cache") and hasattr(m, "probe") for m in model.modules())):
+        return model
+    try:
+        cached = _ADOPTED.get(model)
+    except TypeError:        # not weakly referenceable / not hashable: adopt without remembering
+        cached = None
+    if cached is not None:
+        return cached
+    cfg = getattr(model, "config", None)
+    if cfg is None or not hasattr(model, "state_dict"):
+        raise TypeError(
+            f"generate_ACache on this engine needs an acache_amd model, a ready acache_amd.ModelRunner or a "
+            f"LLaDA / Dream checkpoint model object (with .config and .state_dict()), got {type(model).__name__}")
+    if hasattr(cfg, "d_model"):
+        from .llada import engine_model_from_checkpoint
+    elif hasattr(cfg, "hidden_size"):
+        from .dream import engine_model_from_checkpoint
+    else:
+        raise TypeError(f"generate_ACache: {type(cfg).__name__} is neither a LLaDA nor a Dream configuration")
+    engine = engine_model_from_checkpoint(model)   # TypeError for settings the engine's decoder does not implement
+    try:
+        _ADOPTED[model] = engine
+    except TypeError:
+        pass
+    return engine
+
+
 def _as_runner(model, *, mask_id, block_length, gen_length, anchor_ratio, selection_mode, threshold,
                temperature, remasking, total_len, affix_len) -> ModelRunner:
     if isinstance(model, ModelRunner):
@@ -145,16 +185,7 @@ def _as_runner(model, *, mask_id, block_length, gen_length, anchor_ratio, select
         runner.config.block_length = block_length
         runner.config.gen_length = gen_length
         return runner
-    inner = getattr(model, "model", None)
-    engine_model = (inner is not None and hasattr(model, "config")
-                    and any(hasattr(m, "k_cache") and hasattr(m, "probe") for m in model.modules()))
-    if not engine_model:
-        # an HF checkpoint model attends over dense [B, H, L, D] caches inside its own forward; this entry point
-        # runs on the paged engine and cannot drive it
-        raise TypeError(
-            f"generate_ACache on this engine needs an acache_amd model (acache_amd.llada.LLaDAModelLM, "
-            f"acache_amd.dream.DreamModelLM) or a ready acache_amd.ModelRunner, got {type(model).__name__}: "
-            f"load the checkpoint's weights into the engine model first.")
+    model = _engine_model(model)
     bs = 256
     blocks = 2 * (-(-affix_len // bs)) + -(-(total_len + affix_len) // bs) + 2
     cfg = Config(hf_config=model.config, mask_id=mask_id, recompute_batch_size=1, max_num_seqs=1,

@@ -241,3 +241,90 @@ class LLaDAModelLM(nn.Module):
     def forward(self, input_ids, position_ids=None, logits_keep_indices=None, compute_logits=True):
         return self.model(input_ids, position_ids=position_ids, compute_logits=compute_logits,
                           logits_keep_indices=logits_keep_indices)
+
+
+# ---------------------------------------------------------------------------------------------------
+# Taking over a checkpoint model object
+#
+# The HF path of the reference hands its entry points the checkpoint's own model class
+# (llada/eval_ACache.py:100-107 loads llada/model/modeling_llada.py:LLaDAModelLM in bf16 and passes it to
+# generate_with_anchor_attention, :189).  That class attends over dense [B, H, L, D] caches inside its own
+# forward and cannot run on the paged engine, but its parameters can: this module's blocks use the same
+# parameter names, so the engine model is built around the checkpoint's tensors without copying them.
+
+def _plain(value):
+    """Configuration enums of the checkpoint (StrEnum members) and plain strings compare alike."""
+    value = getattr(value, "value", value)
+    return value.lower() if isinstance(value, str) else value
+
+
+def config_from_checkpoint(cfg) -> LLaDAConfig:
+    """The engine's configuration for a checkpoint configuration (llada/model/configuration_llada.py:154-381).
+    Raises ``TypeError`` naming every setting this decoder stack does not implement."""
+    needed = ("d_model", "n_heads", "n_layers", "vocab_size")
+    if any(not hasattr(cfg, name) for name in needed):
+        raise TypeError(f"not a LLaDA checkpoint configuration: {type(cfg).__name__} lacks one of {needed}")
+    get = lambda name, default=None: getattr(cfg, name, default)
+    wanted = {
+        "rope": True, "alibi": False, "block_type": "llama", "layer_norm_type": "rms", "activation_type": "silu",
+        "include_bias": False, "attention_layer_norm": False, "input_emb_norm": False, "scale_logits": False,
+        "layer_norm_with_affine": True,
+    }
+    problems = [f"{name}={_plain(get(name))!r} (supported: {value!r})" for name, value in wanted.items()
+                if hasattr(cfg, name) and _plain(get(name)) != value]
+    if get("block_group_size", 1) not in (None, 1):
+        problems.append(f"block_group_size={get('block_group_size')} (supported: 1)")
+    if problems:
+        raise TypeError("this engine's LLaDA decoder stack does not implement: " + ", ".join(problems))
+    n_heads = int(cfg.n_heads)
+    if get("n_kv_heads") is not None:
+        n_kv = int(cfg.n_kv_heads)
+    else:
+        n_kv = 1 if get("multi_query_attention") is True else n_heads
+    hidden = get("mlp_hidden_size")
+    if hidden is None:
+        hidden = int(get("mlp_ratio", 4)) * int(cfg.d_model)
+    mask_id = get("mask_token_id")
+    return LLaDAConfig(
+        vocab_size=int(get("embedding_size") or cfg.vocab_size), d_model=int(cfg.d_model), n_heads=n_heads,
+        n_kv_heads=n_kv, n_layers=int(cfg.n_layers), mlp_hidden_size=int(hidden), rope=True,
+        rope_theta=float(get("rope_theta", 10000.0)), max_sequence_length=int(get("max_sequence_length", 1024)),
+        rms_norm_eps=float(get("rms_norm_eps", 1e-5)),
+        mask_token_id=int(mask_id) if mask_id is not None else LLaDAConfig.mask_token_id,
+        weight_tying=bool(get("weight_tying", False)), qkv_bias=bool(get("include_qkv_bias", False)))
+
+
+def _engine_dtype(state):
+    """Parameters as the kernels take them: bf16 / f16 tensors are used as they are (no copy), anything else is
+    converted to bf16."""
+    return {name: t if t.dtype in (torch.bfloat16, torch.float16) or not t.is_floating_point() else t.to(torch.bfloat16)
+            for name, t in state.items()}
+
+
+def adopt_state(engine_cls, config: LLaDAConfig, state: dict):
+    """An ``engine_cls`` model whose parameters ARE the tensors of ``state`` (no second copy of the weights in
+    device memory; the merged projections the blocks build on first use are the only copies)."""
+    with torch.device("meta"):
+        engine = engine_cls(config)
+    state = _engine_dtype(state)
+    tied = config.weight_tying and "model.transformer.ff_out.weight" not in state
+    if tied:  # the checkpoint scores against the embedding matrix (modeling_llada.py: F.linear(x, wte.weight))
+        state = dict(state)
+        state["model.transformer.ff_out.weight"] = state["model.transformer.wte.weight"]
+    engine.load_state_dict(state, strict=True, assign=True)
+    for p in engine.parameters():
+        p.requires_grad_(False)
+    return engine.eval()
+
+
+def engine_model_from_checkpoint(model) -> "LLaDAModelLM":
+    """The engine model for a checkpoint-style LLaDA model object: same configuration, the same parameter tensors.
+    ``model`` needs ``.config`` and ``.state_dict()`` with the checkpoint's names (``model.transformer.blocks.N.*``)."""
+    config = config_from_checkpoint(model.config)
+    state = model.state_dict()
+    if not any(name.startswith("model.transformer.blocks.") for name in state):
+        raise TypeError(f"{type(model).__name__}: no 'model.transformer.blocks.*' parameters in its state dict")
+    try:
+        return adopt_state(LLaDAModelLM, config, state)
+    except RuntimeError as e:  # load_state_dict lists missing / unexpected / mis-shaped entries
+        raise TypeError(f"{type(model).__name__}: its parameters do not fit the engine's LLaDA model: {e}") from e

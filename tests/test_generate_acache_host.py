@@ -97,9 +97,39 @@ def test_coerce_bool_and_ceil():
     assert ceil_to_int(3.0) == 3 and ceil_to_int(3.0000001) == 4 and ceil_to_int(0.07 * 100) == math.ceil(0.07 * 100) == 8
 
 
-def test_foreign_models_are_rejected_with_a_type_error():
-    """The entry points keep the reference's signature but run on the paged engine: a model that is not built from
-    this package's attention modules (an HF checkpoint model, say) is refused before any device work."""
+def _llada_checkpoint_config(**changes):
+    """The fields of llada/model/configuration_llada.py the fixture's model was built with
+    (tests/golden/make_hf_path_vectors.py), as a plain namespace."""
+    from types import SimpleNamespace
+
+    fields = dict(d_model=256, n_heads=2, n_layers=2, mlp_hidden_size=128, vocab_size=64, embedding_size=64,
+                  mask_token_id=63, eos_token_id=0, pad_token_id=0, rope=True, rope_theta=10000.0, alibi=False,
+                  block_type="llama", activation_type="silu", layer_norm_type="rms", rms_norm_eps=1e-5,
+                  include_bias=False, include_qkv_bias=False, weight_tying=False, input_emb_norm=False,
+                  flash_attention=False, max_sequence_length=256, scale_logits=False, n_kv_heads=None,
+                  multi_query_attention=None, mlp_ratio=4)
+    fields.update(changes)
+    return SimpleNamespace(**fields)
+
+
+class CheckpointModelDouble:
+    """Stands where the checkpoint's model object stands in the reference's call (llada/eval_ACache.py:189): a
+    class of another package with ``.config`` and ``.state_dict()`` under the checkpoint's parameter names."""
+
+    def __init__(self, config, state):
+        self.config, self._state = config, state
+
+    def state_dict(self):
+        return self._state
+
+
+def _fixture_weights():
+    from pathlib import Path
+
+    return torch.load(Path(__file__).resolve().parent / "golden" / "hf_path_vectors.pt", weights_only=True)["weights"]
+
+
+def test_objects_that_are_no_checkpoint_model_are_rejected_with_a_type_error():
     from acache_amd.generate_acache import generate_with_anchor_attention
 
     class Foreign(torch.nn.Module):
@@ -109,6 +139,87 @@ def test_foreign_models_are_rejected_with_a_type_error():
             self.config = object()
 
     prompt = torch.arange(2, 10).unsqueeze(0)
-    with pytest.raises(TypeError, match="needs an acache_amd model"):
-        generate_with_anchor_attention(Foreign(), prompt, steps=4, gen_length=4, block_length=4, mask_id=MASK,
-                                       affix_start=0, affix_end=4)
+    args = dict(steps=4, gen_length=4, block_length=4, mask_id=MASK, affix_start=0, affix_end=4)
+    with pytest.raises(TypeError, match="neither a LLaDA nor a Dream configuration"):
+        generate_with_anchor_attention(Foreign(), prompt, **args)
+    with pytest.raises(TypeError, match="checkpoint model object"):
+        generate_with_anchor_attention(object(), prompt, **args)
+    # a LLaDA configuration with settings this decoder stack lacks: every one of them is named
+    odd = CheckpointModelDouble(_llada_checkpoint_config(alibi=True, block_type="sequential"), _fixture_weights())
+    with pytest.raises(TypeError, match=r"alibi=True.*block_type='sequential'"):
+        generate_with_anchor_attention(odd, prompt, **args)
+    # parameters that do not fit the configuration
+    short = CheckpointModelDouble(_llada_checkpoint_config(n_layers=3), _fixture_weights())
+    with pytest.raises(TypeError, match="do not fit"):
+        generate_with_anchor_attention(short, prompt, **args)
+
+
+def test_checkpoint_model_is_adopted_without_copying_its_weights():
+    """The reference's own parameter names (the fixture holds the state dict of llada/model/modeling_llada.py's
+    LLaDAModelLM) load as they are, and the engine model's parameters are those very tensors."""
+    from acache_amd.generate_acache import _engine_model
+    from acache_amd.llada import LLaDAModelLM
+
+    weights = _fixture_weights()
+    checkpoint_model = CheckpointModelDouble(_llada_checkpoint_config(), weights)
+    engine = _engine_model(checkpoint_model)
+    assert isinstance(engine, LLaDAModelLM) and not engine.training
+    cfg = engine.config
+    assert (cfg.d_model, cfg.n_heads, cfg.effective_n_kv_heads, cfg.n_layers, cfg.mlp_hidden_size) == (256, 2, 2, 2, 128)
+    assert (cfg.vocab_size, cfg.mask_token_id, cfg.rope_theta, cfg.max_sequence_length) == (64, 63, 10000.0, 256)
+    state = engine.state_dict()
+    assert set(state) == set(weights)
+    assert all(state[name].data_ptr() == weights[name].data_ptr() for name in weights)
+    assert not any(p.requires_grad for p in engine.parameters())
+    assert _engine_model(checkpoint_model) is engine          # built once per checkpoint object
+    assert _engine_model(engine) is engine                    # an engine model passes through
+    # fp32 weights are converted for the kernels (bf16), tied embeddings score against the embedding matrix
+    tied = {k: v.float() for k, v in weights.items() if k != "model.transformer.ff_out.weight"}
+    engine32 = _engine_model(CheckpointModelDouble(_llada_checkpoint_config(weight_tying=True), tied))
+    assert all(p.dtype == torch.bfloat16 for p in engine32.parameters())
+    head, wte = engine32.model.transformer["ff_out"].weight, engine32.model.transformer["wte"].weight
+    assert head.data_ptr() == wte.data_ptr()
+
+
+def test_dream_checkpoint_names_map_onto_the_engine_model():
+    """dream/model/modeling_dream.py's parameter names (read from its module definitions, :286-343, 624-629,
+    793-799, 945; that model does not construct in this environment, so no state dict of it is on file)."""
+    from types import SimpleNamespace
+
+    from acache_amd import dream
+
+    cfg = dream.DreamConfig(vocab_size=64, d_model=256, n_heads=4, n_kv_heads=2, n_layers=2, mlp_hidden_size=128,
+                            max_sequence_length=128, mask_token_id=63)
+    ours = dream.DreamModelLM(cfg).to(torch.bfloat16)
+    theirs = {}
+    for i in range(2):
+        b = f"model.transformer.blocks.{i}."
+        sd = ours.state_dict()
+        for proj in "qkv":
+            theirs[f"model.layers.{i}.self_attn.{proj}_proj.weight"] = sd[b + f"{proj}_proj.weight"]
+            theirs[f"model.layers.{i}.self_attn.{proj}_proj.bias"] = sd[b + f"{proj}_proj.bias"]
+        theirs[f"model.layers.{i}.self_attn.o_proj.weight"] = sd[b + "attn_out.weight"]
+        theirs[f"model.layers.{i}.mlp.gate_proj.weight"] = sd[b + "ff_proj.weight"]
+        theirs[f"model.layers.{i}.mlp.up_proj.weight"] = sd[b + "up_proj.weight"]
+        theirs[f"model.layers.{i}.mlp.down_proj.weight"] = sd[b + "ff_out.weight"]
+        theirs[f"model.layers.{i}.input_layernorm.weight"] = sd[b + "attn_norm.weight"]
+        theirs[f"model.layers.{i}.post_attention_layernorm.weight"] = sd[b + "ff_norm.weight"]
+    theirs["model.embed_tokens.weight"] = sd["model.transformer.wte.weight"]
+    theirs["model.norm.weight"] = sd["model.transformer.ln_f.weight"]
+    theirs["lm_head.weight"] = sd["model.transformer.ff_out.weight"]
+    theirs["model.rotary_emb.inv_freq"] = torch.zeros(64)           # a buffer the engine does not take
+    hf_cfg = SimpleNamespace(vocab_size=64, hidden_size=256, intermediate_size=128, num_hidden_layers=2,
+                             num_attention_heads=4, num_key_value_heads=2, hidden_act="silu",
+                             max_position_embeddings=128, rms_norm_eps=1e-6, rope_theta=1e6, rope_scaling=None,
+                             use_sliding_window=False, mask_token_id=63, tie_word_embeddings=False)
+    engine = dream.engine_model_from_checkpoint(CheckpointModelDouble(hf_cfg, theirs))
+    assert isinstance(engine, dream.DreamModelLM) and engine.config.qkv_bias and engine.config.effective_n_kv_heads == 2
+    got = engine.state_dict()
+    assert set(got) == set(sd) and all(torch.equal(got[k], sd[k]) for k in sd)
+    hf_cfg.rope_scaling = {"rope_type": "yarn", "factor": 4.0}
+    with pytest.raises(TypeError, match="rope_scaling"):
+        dream.engine_model_from_checkpoint(CheckpointModelDouble(hf_cfg, theirs))
+    hf_cfg.rope_scaling = None
+    theirs["model.layers.0.self_attn.q_norm.weight"] = torch.zeros(4)
+    with pytest.raises(TypeError, match="has no place"):
+        dream.engine_model_from_checkpoint(CheckpointModelDouble(hf_cfg, theirs))

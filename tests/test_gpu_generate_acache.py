@@ -27,21 +27,29 @@ def _model(device, seed=0):
 FIXTURE = Path(__file__).resolve().parent / "golden" / "hf_path_vectors.pt"
 
 
-def _fixture(device):
+def _fixture(device, as_checkpoint_object=False):
     """The reference's own outputs (tests/golden/make_hf_path_vectors.py ran llada/generate_ACache.py on the CPU in
-    fp32 over a 2-layer random model with 2 heads of 128) and this package's model loaded with the same weights."""
+    fp32 over a 2-layer random model with 2 heads of 128) and a model with the same weights: this package's engine
+    model, or a stand-in for the checkpoint model object the reference's caller passes (configuration fields and
+    state dict of llada/model/modeling_llada.py's class, no forward of its own)."""
     data = torch.load(FIXTURE, weights_only=True)
+    if as_checkpoint_object:
+        from .test_generate_acache_host import CheckpointModelDouble, _llada_checkpoint_config
+
+        weights = {name: t.to(device) for name, t in data["weights"].items()}
+        return data["cases"], CheckpointModelDouble(_llada_checkpoint_config(), weights)
     model = LLaDAModelLM(LLaDAConfig(**data["config"]))
     model.load_state_dict(data["weights"])       # same parameter names as the reference's LLaDAModelLM
     return data["cases"], model.to(device=device, dtype=torch.bfloat16).eval()
 
 
-def test_importance_matches_the_reference_fixture(device):
+@pytest.mark.parametrize("as_checkpoint_object", [False, True])
+def test_importance_matches_the_reference_fixture(device, as_checkpoint_object):
     """compute_attention_importance_cross_affix against the values the reference returned for prefix, infix and
     suffix placement.  The reference ran in fp32, the engine in bf16 with the relocation on the query side:
     measured difference 0.044 absolute / 4.6 % relative at most; bound 0.1 / 8 %.  The anchors chosen from the two
     importance vectors must be the same tokens."""
-    cases, model = _fixture(device)
+    cases, model = _fixture(device, as_checkpoint_object)
     for c in cases:
         kw = c["kwargs"]
         cache = tuple((k.to(device), v.to(device)) for k, v in c["affix_cache"])
@@ -55,13 +63,15 @@ def test_importance_matches_the_reference_fixture(device):
                 == G.select_anchor_tokens(want.to(device), k, "top").tolist()), c["name"]
 
 
+@pytest.mark.parametrize("as_checkpoint_object", [False, True])
 @pytest.mark.parametrize("from_cache", [True, False])
-def test_generation_matches_the_reference_fixture(device, from_cache):
+def test_generation_matches_the_reference_fixture(device, from_cache, as_checkpoint_object):
     """generate_with_anchor_attention against the reference's returned sequence and forward count, with the HF-layout
     affix cache the reference was given and with the engine's own affix precompute.  Prompt positions and the
     number of forwards must be equal; of the 8 generated tokens at most one may differ (fp32 there, bf16 here: an
-    arg-max near a tie can flip; measured: none differs)."""
-    cases, model = _fixture(device)
+    arg-max near a tie can flip; measured: none differs).  ``as_checkpoint_object``: the call as the reference's
+    caller makes it, with the checkpoint's model object in the ``model`` argument."""
+    cases, model = _fixture(device, as_checkpoint_object)
     for c in cases:
         kw = dict(c["kwargs"])
         cache = tuple((k.to(device), v.to(device)) for k, v in c["affix_cache"]) if from_cache else None

@@ -153,3 +153,39 @@ def test_batched_engine_applies_the_dream_rule(device):
                      prompt_affix_start=2, prompt_affix_end=18)
     out_f, _ = full.generate_with_acache([seq_f])
     assert sum(a == b for a, b in zip(out_f[0], out_b[0])) >= 6
+
+
+def test_checkpoint_model_object_gives_the_same_tokens(device):
+    """The call as dream/eval_ACache.py makes it: ``model`` is the checkpoint's model object (here a stand-in with
+    dream/model/modeling_dream.py's configuration fields and parameter names around the same weights).  The engine
+    model is built around those tensors and must generate exactly what the engine model itself generates."""
+    from types import SimpleNamespace
+
+    from .test_generate_acache_host import CheckpointModelDouble
+
+    cfg, model = _model(device)
+    sd = model.state_dict()
+    theirs = {"model.embed_tokens.weight": sd["model.transformer.wte.weight"],
+              "model.norm.weight": sd["model.transformer.ln_f.weight"],
+              "lm_head.weight": sd["model.transformer.ff_out.weight"],
+              "model.rotary_emb.inv_freq": torch.zeros(64, device=device)}
+    names = {"self_attn.q_proj": "q_proj", "self_attn.k_proj": "k_proj", "self_attn.v_proj": "v_proj",
+             "self_attn.o_proj": "attn_out", "mlp.gate_proj": "ff_proj", "mlp.up_proj": "up_proj",
+             "mlp.down_proj": "ff_out", "input_layernorm": "attn_norm", "post_attention_layernorm": "ff_norm"}
+    for i in range(cfg.n_layers):
+        for hf, ours in names.items():
+            for leaf in ("weight", "bias"):
+                key = f"model.transformer.blocks.{i}.{ours}.{leaf}"
+                if key in sd:
+                    theirs[f"model.layers.{i}.{hf}.{leaf}"] = sd[key].clone()   # clone: the engine model re-points its own views
+    hf_cfg = SimpleNamespace(vocab_size=64, hidden_size=256, intermediate_size=128, num_hidden_layers=2,
+                             num_attention_heads=4, num_key_value_heads=2, hidden_act="silu",
+                             max_position_embeddings=128, rms_norm_eps=cfg.rms_norm_eps, rope_theta=10000.0,
+                             rope_scaling=None, use_sliding_window=False, mask_token_id=MASK, tie_word_embeddings=False)
+    checkpoint_model = CheckpointModelDouble(hf_cfg, theirs)
+    prompt = torch.tensor([[3, 4] + list(range(20, 36)) + [5, 6]], device=device)
+    kw = dict(steps=8, gen_length=8, block_length=4, mask_id=MASK, anchor_ratio=0.25, affix_start=2, affix_end=18,
+              threshold=0.9)
+    want, nfe_want = GD.generate_with_anchor_attention(model, prompt, **kw)
+    got, nfe_got = GD.generate_with_anchor_attention(checkpoint_model, prompt, **kw)
+    assert nfe_got == nfe_want and torch.equal(got, want)
