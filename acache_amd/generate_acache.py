@@ -24,11 +24,12 @@ the paged engine of this package (``ModelRunner`` + HIP kernels).  Consequences 
 """
 from __future__ import annotations
 
-import weakref
 from typing import Optional, Tuple
 
 import torch
 import torch.nn.functional as F
+
+from .checkpoint import engine_model_for
 
 from . import ops
 from .config import Config
@@ -140,42 +141,6 @@ def get_transfer_index_dynamic(logits, temperature, remasking, mask_index, x, nu
 
 
 # ------------------------------------------------------------------------------------------ engine glue
-_ADOPTED = weakref.WeakKeyDictionary()   # checkpoint model object -> the engine model built around its weights
-
-
-def _engine_model(model):
-    """``model`` itself when it is one of this package's models; for the checkpoint model object the HF path
-    passes (llada/eval_ACache.py:100-107, 189; dream/eval_ACache.py likewise), the engine model built around the
-    same parameter tensors, made once per object."""
-    inner = getattr(model, "model", None)
-    if (inner is not None and hasattr(model, "config")
-            and any(hasattr(m, "k_cache") and hasattr(m, "probe") for m in model.modules())):
-        return model
-    try:
-        cached = _ADOPTED.get(model)
-    except TypeError:        # not weakly referenceable / not hashable: adopt without remembering
-        cached = None
-    if cached is not None:
-        return cached
-    cfg = getattr(model, "config", None)
-    if cfg is None or not hasattr(model, "state_dict"):
-        raise TypeError(
-            f"generate_ACache on this engine needs an acache_amd model, a ready acache_amd.ModelRunner or a "
-            f"LLaDA / Dream checkpoint model object (with .config and .state_dict()), got {type(model).__name__}")
-    if hasattr(cfg, "d_model"):
-        from .llada import engine_model_from_checkpoint
-    elif hasattr(cfg, "hidden_size"):
-        from .dream import engine_model_from_checkpoint
-    else:
-        raise TypeError(f"generate_ACache: {type(cfg).__name__} is neither a LLaDA nor a Dream configuration")
-    engine = engine_model_from_checkpoint(model)   # TypeError for settings the engine's decoder does not implement
-    try:
-        _ADOPTED[model] = engine
-    except TypeError:
-        pass
-    return engine
-
-
 def _as_runner(model, *, mask_id, block_length, gen_length, anchor_ratio, selection_mode, threshold,
                temperature, remasking, total_len, affix_len) -> ModelRunner:
     if isinstance(model, ModelRunner):
@@ -185,7 +150,7 @@ def _as_runner(model, *, mask_id, block_length, gen_length, anchor_ratio, select
         runner.config.block_length = block_length
         runner.config.gen_length = gen_length
         return runner
-    model = _engine_model(model)
+    model = engine_model_for(model)
     bs = 256
     blocks = 2 * (-(-affix_len // bs)) + -(-(total_len + affix_len) // bs) + 2
     cfg = Config(hf_config=model.config, mask_id=mask_id, recompute_batch_size=1, max_num_seqs=1,

@@ -33,6 +33,7 @@ import torch
 
 from . import ops
 from .block_manager import BlockManager
+from .checkpoint import engine_model_for
 from .sequence import DeviceLayout, Sequence
 from .utils import add_gumbel_noise, get_context, reset_context, set_context
 
@@ -40,6 +41,12 @@ from .utils import add_gumbel_noise, get_context, reset_context, set_context
 class ModelRunner:
     def __init__(self, model, config):
         self.config = config
+        # the reference's caller passes its own model class (model_runner.py:15-19); a model that is not built from
+        # this package's blocks is taken over: same parameter tensors under the engine's decoder stack
+        unwrapped = model.module if hasattr(model, "module") else model
+        engine = engine_model_for(unwrapped)
+        if engine is not unwrapped:
+            model = engine
         self.model = model
         self.base_model = model.module if hasattr(model, "module") else model
         self.device = model.device

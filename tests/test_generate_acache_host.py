@@ -157,7 +157,7 @@ def test_objects_that_are_no_checkpoint_model_are_rejected_with_a_type_error():
 def test_checkpoint_model_is_adopted_without_copying_its_weights():
     """The reference's own parameter names (the fixture holds the state dict of llada/model/modeling_llada.py's
     LLaDAModelLM) load as they are, and the engine model's parameters are those very tensors."""
-    from acache_amd.generate_acache import _engine_model
+    from acache_amd.checkpoint import engine_model_for as _engine_model
     from acache_amd.llada import LLaDAModelLM
 
     weights = _fixture_weights()

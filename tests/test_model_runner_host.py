@@ -209,3 +209,21 @@ def test_requests_longer_than_the_rotary_table_are_refused():
     with pytest.raises(ValueError, match="rotary table"):
         runner.generate_with_dual_cache([too_long])
     assert runner.model.calls == 0
+
+
+def test_model_runner_takes_over_a_checkpoint_model_object():
+    """``ModelRunner(model, config)`` with the model class of another package (the reference's caller passes its
+    own, model_runner.py:15-19): the runner runs the engine model built around the same parameter tensors."""
+    from .test_generate_acache_host import CheckpointModelDouble, _fixture_weights, _llada_checkpoint_config
+
+    weights = _fixture_weights()
+    checkpoint_model = CheckpointModelDouble(_llada_checkpoint_config(), weights)
+    serve = Config(hf_config=checkpoint_model.config, mask_id=63, recompute_batch_size=2, gen_length=4, block_length=4,
+                   cache_block_size=8, num_kvcache_blocks=2, temperature=0.0, threshold=0.0)
+    runner = ModelRunner(checkpoint_model, serve)
+    assert isinstance(runner.model, LLaDAModelLM) and runner.base_model is runner.model
+    q = runner._llada_blocks()[0].q_proj.weight
+    assert q.data_ptr() == weights["model.transformer.blocks.0.q_proj.weight"].data_ptr()
+    assert runner.kv_cache.shape == (2, 2, 2, 8, 2, 128)      # [K/V, layers, blocks, block size, KV heads, head dim]
+    with pytest.raises(TypeError, match="checkpoint model object"):
+        ModelRunner(object(), serve)
