@@ -160,6 +160,20 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
     qo_bytes = 2 * total_q * H * D * 2
     tflops = flops / (avg_ms * 1e-3) / 1e12
     extra = {"cpu_baseline": cpu_attention_baseline(torch, q, kc, vc, w)} if cpu_baseline else {}
+    # the same kernel on a batch without raggedness (4 requests x 4096 queries x 4096 keys, distinct rows): what its
+    # inner loop reaches when every query tile is full and all units are equal (reported, not used in `frac`)
+    ub, un = 4, 4096
+    uq = (torch.randn(ub * un, H, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    uk = (torch.randn(ub * un // BS, BS, Hkv, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    uv = (torch.randn(ub * un // BS, BS, Hkv, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
+    ucu = torch.arange(0, (ub + 1) * un, un, dtype=torch.int32, device=device)
+    uslots = torch.arange(ub * un, dtype=torch.int32, device=device)
+    for _ in range(3):
+        ops.acache_attention(uq, uk, uv, ucu, ucu, uslots)
+    torch.cuda.synchronize()
+    uni_ms = _event_times_ms(lambda: ops.acache_attention(uq, uk, uv, ucu, ucu, uslots), 7, torch)
+    uniform_tflops = 4 * H * D * ub * un * un / (statistics.median(uni_ms) * 1e-3) / 1e12
+    del uq, uk, uv
     # what the library GEMM reaches on a large square bf16 product on the same box: the practical matrix-core
     # reference next to the nominal peak (reported, not used in `frac`)
     n = 8192
@@ -183,7 +197,8 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
                      "kernel": "varlen_attn_unit_kernel<bf16,128,plain>", "algorithmic_flops": flops,
                      "algorithmic_bytes": kv_bytes + qo_bytes,
                      "achieved_GBps": round((kv_bytes + qo_bytes) / (avg_ms * 1e-3) / 1e9, 1),
-                     "library_gemm_8192_TFLOPs": round(gemm_tflops, 1)},
+                     "library_gemm_8192_TFLOPs": round(gemm_tflops, 1),
+                     "same_kernel_uniform_4x4096x4096_TFLOPs": round(uniform_tflops, 1)},
     }
 
 
