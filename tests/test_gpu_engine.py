@@ -362,36 +362,42 @@ def test_batched_probe_at_admission_selects_the_same_anchors(device, placement, 
     assert all(len(a) == 5 for a in results[0][0])          # ceil(0.4 * 12) anchors per request
 
 
-def test_device_layouts_equal_the_host_layouts(device):
+@pytest.mark.parametrize("ratio,expected_anchors", [(0.4, 5), (0.0, 0), (1.0, 12)])
+def test_device_layouts_equal_the_host_layouts(device, ratio, expected_anchors):
     """Batched serving keeps anchors and slot maps on the device.  What the layout launch produced for the admitted
     requests must be, list for list, what ``Sequence.finalize_slot_mapping`` builds on the host from the same
-    anchors and block tables, and the packed read order must be the host's query-relocation order."""
+    anchors and block tables, and the packed read order must be the host's query-relocation order.  Prefix, infix
+    and suffix placement (generation window in front of the affix); no anchors, some, and all of the affix."""
     cfg, model = _model(device, seed=3)
     affix = list(range(20, 32))
 
     def make(i):
+        if i == 4:   # suffix: [head, window of 4 masks, affix]
+            return Sequence([2, 3] + [63] * 4 + affix, gen_length=4, block_length=4, cache_block_size=8, mask_id=63,
+                            prompt_affix_start=6, prompt_affix_end=6 + len(affix), generation_start=2)
         if i % 2:
             return Sequence(affix + [40 + i, 41 + i], gen_length=4, block_length=4, cache_block_size=8, mask_id=63,
                             prompt_affix_len=len(affix))
         return Sequence([2 + i] * (1 + i) + affix + [40 + i], gen_length=4, block_length=4, cache_block_size=8,
                         mask_id=63, prompt_affix_start=1 + i, prompt_affix_end=1 + i + len(affix))
 
-    runner = ModelRunner(model, _serve(cfg, max_num_seqs=0, num_kvcache_blocks=40, anchor_ratio=0.4))
-    seqs = [make(i) for i in range(4)]
+    runner = ModelRunner(model, _serve(cfg, max_num_seqs=0, num_kvcache_blocks=48, anchor_ratio=ratio))
+    seqs = [make(i) for i in range(5)]
     with torch.inference_mode():
         prefix = runner._prepare_acache(seqs)
         batch = []
-        assert runner._admit_sequences_with_acache(batch, seqs, prefix, True) == 4
+        assert runner._admit_sequences_with_acache(batch, seqs, prefix, True) == 5
     for seq in seqs:
         layout = seq.device_layout
         assert layout is not None and layout.anchors.dtype == torch.int32
         twin = Sequence(seq.token_ids[: seq.num_prompt_tokens], gen_length=4, block_length=4, cache_block_size=8,
-                        mask_id=63, prompt_affix_start=seq.affix_start, prompt_affix_end=seq.affix_end)
-        twin.enable_acache(len(affix), 0.4, affix_start=seq.affix_start, affix_end=seq.affix_end)
+                        mask_id=63, prompt_affix_start=seq.affix_start, prompt_affix_end=seq.affix_end,
+                        generation_start=seq.generation_start if seq.generation_start < seq.affix_start else None)
+        twin.enable_acache(len(affix), ratio, affix_start=seq.affix_start, affix_end=seq.affix_end)
         twin.set_anchor_positions(layout.anchors.tolist())
         twin.block_table = list(seq.block_table)
         twin.finalize_slot_mapping()
-        assert seq.anchor_positions == twin.anchor_positions and len(twin.anchor_positions) == 5
+        assert seq.anchor_positions == twin.anchor_positions and len(twin.anchor_positions) == expected_anchors
         assert seq.read_slot_map == twin.read_slot_map
         assert seq.recompute_positions == twin.recompute_positions
         assert seq.recompute_slot_mapping == twin.recompute_slot_mapping
