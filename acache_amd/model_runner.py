@@ -750,10 +750,6 @@ class ModelRunner:
                     self._to_device(slot_mapping, torch.int32), block_tables, total_k=int(seqlens.sum()))
         return self._to_device(positions, torch.int64)
 
-    def _acache_read_side(self, group):
-        relocation_materialized = all(getattr(s, "relocated_affix_materialized", False) for s in group)
-        return relocation_materialized
-
     def prepare_caching_acache(self, seqs, active_indices=None, use_query_relocation=None):
         """Cache refresh with affix reuse: queries = anchors + non-affix tokens; keys read through ``read_slot_map``."""
         group = self._select(seqs, active_indices)
@@ -916,7 +912,7 @@ class ModelRunner:
         assert step > 0, "recompute_batch_size must be larger than 0"
         max_num_seqs = cfg.max_num_seqs if cfg.max_num_seqs > 0 else len(prompts)
         use_acache = prefix is not None
-        dream = str(getattr(cfg, "model_type", "")).lower() == "dream"
+        dream = self._is_dream_model()
         if timing is None:
             timing = self._new_timing(mode, len(prompts))
         self.last_timing = timing or {}
