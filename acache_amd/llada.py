@@ -295,9 +295,9 @@ def config_from_checkpoint(cfg) -> LLaDAConfig:
 
 
 def _engine_dtype(state):
-    """Parameters as the kernels take them: bf16 / f16 tensors are used as they are (no copy), anything else is
-    converted to bf16."""
-    return {name: t if t.dtype in (torch.bfloat16, torch.float16) or not t.is_floating_point() else t.to(torch.bfloat16)
+    """Parameters as the engine takes them: its paged cache is bf16 (as the reference's, model_runner.py:206-208), so
+    bf16 tensors are used as they are (no copy) and any other floating type is converted to bf16."""
+    return {name: t if t.dtype == torch.bfloat16 or not t.is_floating_point() else t.to(torch.bfloat16)
             for name, t in state.items()}
 
 
