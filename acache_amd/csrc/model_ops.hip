@@ -32,7 +32,9 @@ __global__ __launch_bounds__(256) void swiglu_kernel(char *out, const char *gu, 
 }
 
 // sum[t, :] = x[t, :] + delta[t, :] (rounded to the storage type),
-// y[t, :]   = sum[t, :] * rsqrt(mean(sum[t, :]^2) + eps) * w[:], statistics in fp32, one rounding of y.
+// y[t, :]   = round(sum[t, :] * rsqrt(mean(sum[t, :]^2) + eps)) * w[:]: statistics in fp32, the normalised value
+// rounded to the storage type before the weight multiplies it and the product rounded again, which is where the
+// reference's layer norm rounds (llada/model/modeling_llada.py:338-350: x.to(og_dtype), then weight * x).
 // Without delta the sum is x itself and is not written.  One 256-thread block per row; a thread keeps its
 // chunks of the row in registers between the two steps (rows of up to 256 * 16 bytes * kMaxChunks).
 constexpr int kMaxChunks = 4;
@@ -83,7 +85,10 @@ __global__ __launch_bounds__(256) void add_rms_norm_kernel(char *sum, const char
       float w[VEC], o[VEC];
       E::unpack(load16(weight + c * 16), w);
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) o[j] = v[i][j] * scale * w[j];
+      for (int j = 0; j < VEC; ++j) o[j] = v[i][j] * scale;
+      E::unpack(E::pack(o), o);  // the normalised row in the storage type
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) o[j] *= w[j];
       store16(yr + c * 16, E::pack(o));
     }
   }

@@ -57,8 +57,11 @@ class RMSNorm(nn.Module):
         self.eps = eps
 
     def forward(self, x):
-        # one fused kernel; statistics and scaling in fp32, one rounding to the activation type
-        return F.rms_norm(x, (x.shape[-1],), self.weight.to(x.dtype), self.eps)
+        # statistics in fp32; the normalised value is rounded to the activation type before the weight multiplies
+        # it, as in the reference (llada/model/modeling_llada.py:338-350) and in ops.add_rms_norm
+        xf = x.float()
+        y = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps)).to(x.dtype)
+        return self.weight.to(x.dtype) * y
 
 
 class RotaryEmbedding(nn.Module):

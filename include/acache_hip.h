@@ -404,8 +404,9 @@ int acache_varlen_attn(
  *
  * acache_add_rms_norm: sum[t, :] = x[t, :] + delta[t, :] rounded to `dtype` (sum may be x itself;
  * with delta == NULL the sum is x and nothing is written to `sum`, which may then be NULL),
- * y[t, :] = sum[t, :] * rsqrt(mean(sum[t, :]^2) + eps) * weight[:], statistics in fp32, one
- * rounding of y.  y may not overlap the other rows.  d * sizeof(dtype) a multiple of 16 and at
+ * y[t, :] = round(sum[t, :] * rsqrt(mean(sum[t, :]^2) + eps)) * weight[:], statistics in fp32, the
+ * normalised value rounded to `dtype` before the weight multiplies it (where the reference's RMS
+ * layer norm rounds, llada/model/modeling_llada.py:338-350), the product rounded again.  y may not overlap the other rows.  d * sizeof(dtype) a multiple of 16 and at
  * most 16 KiB.
  */
 int acache_swiglu(void *out, const void *gate_up, int64_t M, int64_t m,
