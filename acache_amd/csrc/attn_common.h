@@ -223,12 +223,14 @@ __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], floa
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16));
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const float mxc = mx * c;
     // decided per tile of 16 queries, so a query row's arithmetic does not depend on which other rows share
-    // its wave (workgroups may give a wave one or two such tiles)
-    if (__builtin_amdgcn_ballot_w64(mxc > m_run[qt] + 8.0f) != 0) {
+    // its wave (workgroups may give a wave one or two such tiles).  Every lane tests the maximum of its own
+    // keys: the ballot is true exactly when some query's maximum over the whole tile exceeds the bound, so the
+    // cross-lane maximum (two LDS round trips) is only taken when the reference really moves.
+    if (__builtin_amdgcn_ballot_w64(mx * c > m_run[qt] + 8.0f) != 0) {
+      mx = fmaxf(mx, __shfl_xor(mx, 16));
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float mxc = mx * c;
       const float m_new = fmaxf(m_run[qt], mxc);
       const float m_use = m_new == -INFINITY ? 0.0f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
@@ -254,7 +256,8 @@ __device__ __forceinline__ void softmax_probs_slab(const f32x4 (&s_acc)[NQ16][NT
     const float mc = m_run[qt];
     float e[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s_acc[qt][2 * S + (j >> 2)][j & 3] * c - mc);
+    // one fused multiply-add per score (contraction is switched off for this library, so it is asked for by name)
+    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[qt][2 * S + (j >> 2)][j & 3], c, -mc));
     pf[qt][S].w[0] = M::pack2(e[0], e[1]);
     pf[qt][S].w[1] = M::pack2(e[2], e[3]);
     pf[qt][S].w[2] = M::pack2(e[4], e[5]);

@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void importance_stats_kernel(ImportanceParams 
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(sc[u][nt][i] * c - m_new);
+          for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(__builtin_fmaf(sc[u][nt][i], c, -m_new));
         l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + add;
         m_run[qt] = m_new;
       }
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(256) void importance_colsum_kernel(ImportanceParams
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(sc[nt][i] * c - ref);
+        for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(__builtin_fmaf(sc[nt][i], c, -ref));
     }
   };
   vec16 q_a[NR][KS], q_b[NR][KS];
@@ -463,7 +463,7 @@ __global__ __launch_bounds__(256) void importance_stats_lds_kernel(ImportancePar
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(sc[u][nt][i] * c - m_new);
+            for (int i = 0; i < 4; ++i) add += __builtin_amdgcn_exp2f(__builtin_fmaf(sc[u][nt][i], c, -m_new));
           l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + add;
           m_run[qt] = m_new;
         }
@@ -569,7 +569,7 @@ __global__ __launch_bounds__(256) void importance_colsum_lds_kernel(ImportancePa
 #pragma unroll
         for (int nt = 0; nt < 4; ++nt)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(sc[nt][i] * c - ref);
+          for (int i = 0; i < 4; ++i) col[nt][i] += __builtin_amdgcn_exp2f(__builtin_fmaf(sc[nt][i], c, -ref));
       }
     }
 #pragma unroll
