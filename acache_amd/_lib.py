@@ -63,8 +63,7 @@ SIGNATURES = {
         c_int32, c_int64, c_int64,
         c_int32, c_int32, c_int32, c_int32, c_int64,
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
-        c_void_p, c_int64, c_void_p]),
-    "acache_varlen_attn_workspace_bytes": (c_int64, []),
+        c_void_p]),
 }
 
 

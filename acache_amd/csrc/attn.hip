@@ -847,17 +847,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
 }
 
 template <int DTYPE, int D, int NQ16>
-static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, void *workspace, int64_t workspace_bytes,
-                       hipStream_t stream) {
+static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStream_t stream) {
   AttnParams p = p0;
-  // One 4-wave workgroup per (request, 128-row query tile, head) is the default.  The 8-wave persistent kernel
-  // (attn_wide.hip) is faster on batches of equal requests with 129 .. 256 query rows (17 - 22 % measured) and
-  // slower on ragged ones (it runs one workgroup per CU, so the start-up and wind-down of every part it is
-  // dealt are exposed instead of hidden behind a second workgroup): it is taken only when the caller asks for
-  // it with ACACHE_ATTN_WIDE=1 in the environment.
-  static const bool wide_opt_in = [] { const char *e = getenv("ACACHE_ATTN_WIDE"); return e && e[0] == '1'; }();
-  if (wide_opt_in && mode != MODE_KEY_SIDE && total_q > (int64_t)128 * p.B)
-    return launch_attn_wide(p, DTYPE, D, mode, workspace, workspace_bytes, stream);
+  // One 4-wave workgroup per (request, 128-row query tile, head), two workgroups per CU.
   p.num_tiles = (int32_t)((total_q + 127) / 128) + p.B;
   const int64_t blocks = attn_grid_blocks(p);
   if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
@@ -900,8 +892,6 @@ static int launch_attn_any_head_dim(const AttnParams &p0, int mode, int64_t tota
 
 using namespace acache;
 
-extern "C" int64_t acache_varlen_attn_workspace_bytes(void) { return attn_wide_workspace_bytes(); }
-
 extern "C" int acache_varlen_attn(
     void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *cu_q,
     const int32_t *cu_k, const int32_t *slot_map, float scale, int32_t shared_prefix_len,
@@ -909,7 +899,7 @@ extern "C" int acache_varlen_attn(
     const float *rope_sin, int32_t rope_rows, int32_t B, int64_t total_q, int64_t total_k, int32_t H,
     int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t q_token_stride,
     int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t kv_slot_stride,
-    int64_t kv_head_stride, void *workspace, int64_t workspace_bytes, void *stream) {
+    int64_t kv_head_stride, void *stream) {
   if (dtype != ACACHE_BF16 && dtype != ACACHE_F16)
     return fail(ACACHE_E_DTYPE, "varlen_attn: dtype %d not supported (bf16 or f16)", dtype);
   if (D < 16 || D > 256 || D % 16 != 0)
@@ -927,8 +917,6 @@ extern "C" int acache_varlen_attn(
   if (relocate && (!rope_cos || !rope_sin || rope_rows <= 0))
     return fail(ACACHE_E_MODE, "varlen_attn: relocation requested without RoPE tables");
   const int es = 2;
-  if (workspace_bytes < 0 || (workspace && !aligned16(workspace)))
-    return fail(ACACHE_E_ALIGN, "varlen_attn: workspace must be 16-byte aligned, its size non-negative");
   if (!aligned16(out) || !aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) ||
       (q_token_stride * es) % 16 || (q_head_stride * es) % 16 || (out_token_stride * es) % 16 ||
       (out_head_stride * es) % 16 || (kv_slot_stride * es) % 16 || (kv_head_stride * es) % 16)
@@ -946,11 +934,10 @@ extern "C" int acache_varlen_attn(
   p.q_token_bytes = q_token_stride * es; p.q_head_bytes = q_head_stride * es;
   p.o_token_bytes = out_token_stride * es; p.o_head_bytes = out_head_stride * es;
   p.kv_slot_bytes = kv_slot_stride * es; p.kv_head_bytes = kv_head_stride * es;
-  p.ws_slots = nullptr; p.ws_counters = nullptr;
   const int mode = query_side ? MODE_QUERY_SIDE : (relocate ? MODE_KEY_SIDE : MODE_PLAIN);
   hipStream_t st = (hipStream_t)stream;
 #define ACACHE_ATTN(DT, DD) \
-  if (dtype == DT && D == DD) return launch_attn<DT, DD, 2>(p, mode, total_q, workspace, workspace_bytes, st);
+  if (dtype == DT && D == DD) return launch_attn<DT, DD, 2>(p, mode, total_q, st);
   ACACHE_ATTN(ACACHE_BF16, 128)
   ACACHE_ATTN(ACACHE_BF16, 64)
   ACACHE_ATTN(ACACHE_F16, 128)

@@ -38,10 +38,6 @@ struct AttnParams {
   int64_t q_token_bytes, q_head_bytes;
   int64_t o_token_bytes, o_head_bytes;
   int64_t kv_slot_bytes, kv_head_bytes;
-  // persistent schedule: partial-state slots and arrival counters of units dealt to several workgroups
-  // (NULL: units are never split)
-  char *ws_slots;
-  int32_t *ws_counters;
 };
 
 // Which (request, query tile) does global tile index `tile` address?  Lane i loads
@@ -265,10 +261,5 @@ __device__ __forceinline__ void softmax_probs_slab(const f32x4 (&s_acc)[NQ16][NT
     l_acc[qt] = M::run(ones, pf[qt][S], l_acc[qt]);
   }
 }
-
-// 8-wave persistent kernel for requests with more than 128 query rows (attn_wide.hip)
-int64_t attn_wide_workspace_bytes();
-int launch_attn_wide(const AttnParams &p, int dtype, int D, int mode, void *workspace, int64_t workspace_bytes,
-                     hipStream_t stream);
 
 }  // namespace acache

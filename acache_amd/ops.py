@@ -558,29 +558,6 @@ def block_table_slots(
     return out
 
 
-_ATTN_WORKSPACES: dict = {}
-# same switch as the library reads: the 8-wave persistent kernel is taken only on request
-_ATTN_WIDE = os.environ.get("ACACHE_ATTN_WIDE", "")[:1] == "1"
-
-
-def attention_workspace(device) -> torch.Tensor:
-    """The zero-initialised scratch ``acache_varlen_attn`` shares between the parts of a unit that its persistent
-    schedule cut between workgroups: one buffer per (device, stream), allocated on first use and kept.  The
-    kernel leaves the arrival counters at zero, so the buffer is never cleared again."""
-    device = torch.device(device)
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    key = (index, torch.cuda.current_stream(index).cuda_stream)
-    ws = _ATTN_WORKSPACES.get(key)
-    if ws is None:
-        with torch.cuda.device(index):
-            need = int(_lib.load().acache_varlen_attn_workspace_bytes())
-        if need <= 0:
-            raise _lib.AcacheLibraryError("acache_varlen_attn_workspace_bytes failed")
-        ws = torch.zeros(need, dtype=torch.uint8, device=torch.device("cuda", index))
-        _ATTN_WORKSPACES[key] = ws
-    return ws
-
-
 def _varlen_attn(q, k_cache, v_cache, cu_q, cu_k, slots, scale, shared_prefix_len,
                  shared_kv_lens, affix_shifts, cos, sin):
     total_q, H, D = q.shape
@@ -600,15 +577,13 @@ def _varlen_attn(q, k_cache, v_cache, cu_q, cu_k, slots, scale, shared_prefix_le
     B = cu_q.numel() - 1
     rope_rows = 0 if cos is None else cos.shape[0]
     lib = _lib.load()
-    ws = attention_workspace(q.device) if _ATTN_WIDE else None  # only the opt-in 8-wave kernel cuts units
     with torch.cuda.device(q.device):
         rc = lib.acache_varlen_attn(
             _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(cu_q), _ptr(cu_k), _ptr(slots),
             float(scale), int(shared_prefix_len), _ptr(shared_kv_lens), _ptr(affix_shifts),
             _ptr(cos), _ptr(sin), rope_rows,
             B, total_q, slots.numel(), H, Hkv, D, _code(q), num_slots,
-            q.stride(0), q.stride(1), out.stride(0), out.stride(1), slot_stride, head_stride,
-            _ptr(ws), ws.numel() if ws is not None else 0, _stream(q))
+            q.stride(0), q.stride(1), out.stride(0), out.stride(1), slot_stride, head_stride, _stream(q))
     _lib.check(rc, "acache_attention")
     return out
 

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define ACACHE_ABI_VERSION 2
+#define ACACHE_ABI_VERSION 3
 
 /* element types of K/V/Q payloads */
 #define ACACHE_BF16 0
@@ -360,22 +360,8 @@ int acache_build_slot_layout(
  * Schedule (head_dim 64 / 128).  One workgroup of four waves per (request, 128-row query tile, head)
  * unit, two workgroups per CU, units handed out longest request first; K/V tiles of 64 keys reach LDS
  * through the copy engine.  In key-side mode the rows of a tile that lie in shared slots are re-rotated
- * in LDS after they land.  This schedule needs no workspace: pass NULL and 0.
- *
- * workspace / workspace_bytes are read only by an alternative schedule that the library takes when the
- * environment holds ACACHE_ATTN_WIDE=1 (read once per process): eight waves per workgroup on 256-row
- * units, one persistent workgroup per CU, the units laid end to end and cut into equal stretches of
- * key-tile steps.  The parts of a cut unit meet in `workspace`: device memory of at least
- * acache_varlen_attn_workspace_bytes() bytes (a function of the current device's CU count: arrival
- * counters followed by two partial-state slots per workgroup), 16-byte aligned, owned by the caller.
- * Its counters must be ZERO before the first call that uses it (clear the buffer once after
- * allocating it); every call leaves them zero again.  Calls that may overlap in time (different
- * streams) need different workspaces.  The merge order is fixed, so results are bit-identical from
- * run to run; against the default schedule they differ by the rounding of the merge.  With
- * workspace == NULL (or too small) that schedule deals units whole.  It is faster on uniform
- * batches of long requests and slower on ragged ones, which is why it is not the default.
+ * in LDS after they land.  No workspace: the kernel allocates nothing and keeps no state between calls.
  */
-int64_t acache_varlen_attn_workspace_bytes(void);
 int acache_varlen_attn(
     void *out, const void *q, const void *k_cache, const void *v_cache,
     const int32_t *cu_q, const int32_t *cu_k, const int32_t *slot_map,
@@ -386,8 +372,7 @@ int acache_varlen_attn(
     int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
     int64_t q_token_stride, int64_t q_head_stride,
     int64_t out_token_stride, int64_t out_head_stride,
-    int64_t kv_slot_stride, int64_t kv_head_stride,
-    void *workspace, int64_t workspace_bytes, void *stream);
+    int64_t kv_slot_stride, int64_t kv_head_stride, void *stream);
 
 /*
  * Two elementwise steps of the decoder block on either side of the attention path, for
