@@ -651,11 +651,14 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   // Every shared row has its own shift n - slot; in the engine's layouts all shared rows of a request have the
   // shift the caller also passes per request, so the cos / sin rows of that shift are kept in LDS (lds_rope,
   // filled below) and only rows with another shift fetch their own rows from the table.  The row's slot is
-  // fetched one tile ahead (rot_slot), behind the compute phase of the tile before.
+  // fetched one tile ahead (rot_slot), behind the compute phase of the tile before.  A thread's row is one of
+  // the rows its own wave copied (tid / 4 lies in the wave's 16 rows), so the rotation starts as soon as the
+  // wave's own copies have landed and the barrier that publishes the tile publishes the rotated rows.
   constexpr int PAIRS = CH / 2;                    // (d, d + D/2) chunk pairs per row
   constexpr int PER_THREAD = BN * PAIRS / THREADS;  // 2 (D = 128, 4 waves)
   static_assert(BN * PAIRS % THREADS == 0 && PER_THREAD >= 1, "one or more chunk pairs per thread");
   const int rot_row = tid / (PAIRS / PER_THREAD);
+  static_assert(64 / (PAIRS / PER_THREAD) == WAVE_ROWS, "a wave rotates exactly the rows it copies");
   int shift0 = 0;
   if (MODE == MODE_KEY_SIDE) {
     shift0 = p.affix_shifts[b];
@@ -663,7 +666,8 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     if (tid < 2 * D / 4) {  // cos row, then sin row: D floats each, 16 bytes per thread
       const float *src = (tid < D / 4 ? p.cos_tab : p.sin_tab) + (int64_t)shift0 * D + (tid % (D / 4)) * 4;
       store16(lds_rope + tid * 4, load16(src));
-    }  // published by the barrier that publishes the first tile
+    }
+    __syncthreads();  // the first rotation reads these rows before the first tile's barrier
   }
   auto rot_prefetch = [&](int t) __attribute__((always_inline)) {
     const int n = t * BN + rot_row;
@@ -692,7 +696,6 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
       if (delta == shift0) rotate_with(lds_rope, lds_rope + D, 1.0f);
       else rotate_with(p.cos_tab + (int64_t)ad * D, p.sin_tab + (int64_t)ad * D, delta < 0 ? -1.0f : 1.0f);
     }
-    __syncthreads();  // the rotated rows are in place for everybody
   };
   int rot_slot = rot_prefetch(t_begin);
 
@@ -709,12 +712,12 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   for (int t = t_begin; t < t_stop; t += 2) {
     // first tile of the pair: wait for its copies, publish it, start the second, compute
     __builtin_amdgcn_s_waitcnt(0);  // this wave's copies of tile t have landed
-    __syncthreads();                // ... and everybody else's; buffer 1 is no longer being read
     if (MODE == MODE_KEY_SIDE) {
       const int cur = rot_slot;
       rot_slot = rot_prefetch(t + 1);
       rotate_shared_rows(lds_k0, t, cur);
     }
+    __syncthreads();                // ... and everybody else's; buffer 1 is no longer being read
     bool stepped = false;
     if (t + 1 < t_end) {
       load_slots(t + 2, slot_a);    // slot loads go first: vmcnt retires in order, so waiting
@@ -731,12 +734,12 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     }
     if (t + 1 >= t_stop) break;
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
     if (MODE == MODE_KEY_SIDE) {
       const int cur = rot_slot;
       rot_slot = rot_prefetch(t + 2);
       rotate_shared_rows(lds_k1, t + 1, cur);
     }
+    __syncthreads();
     stepped = false;
     if (t + 2 < t_end) {
       load_slots(t + 3, slot_b);
@@ -754,9 +757,9 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   }
   if (PEEL_TAIL && t_stop < t_end) {  // tail tile t_stop: its copies were issued one step earlier
     __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
     const bool odd = ((t_stop - t_begin) & 1) != 0;
     if (MODE == MODE_KEY_SIDE) rotate_shared_rows(odd ? lds_k1 : lds_k0, t_stop, rot_slot);
+    __syncthreads();
     if (nq_valid > 0)
       compute.template operator()<true>(odd ? lds_k1 : lds_k0, odd ? lds_v1 : lds_v0, kv_len - t_stop * BN, false,
                                         nullptr, nullptr, slot_a);
