@@ -380,7 +380,36 @@ def attention_shape_sweep(torch, device, ops, steps):
         kv_bytes = 2 * S * Hkv * D * 2
         rows.append({"B": B, "q": q, "kv": kv, "H": H, "H_kv": Hkv, "us": round(ms * 1e3, 1),
                      "TFLOPs": round(4 * H * D * B * q * kv / ms / 1e9, 0), "kv_GBps": round(kv_bytes / ms / 1e6, 0)})
-    print(json.dumps({"attention_shape_sweep": rows}))
+    # The three relocation modes on one relocated anchor-recompute shape: batch 16, 232 queries and 1 400 keys per
+    # request, a shared affix of 1 000 slots placed 50 + 10 b positions into request b (back-to-back launches).
+    from acache_amd.rope import rope_table
+    B, H, A, R, q_per = 16, 32, 1000, 400, 232
+    S = A + B * R + 64
+    K = (torch.randn(S, 1, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+    V = torch.randn(S, 1, H, D, device=device).to(torch.bfloat16)
+    Q = (torch.randn(B * q_per, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+    cos, sin = (t.to(device) for t in rope_table(2048, D, 5e5))
+    shared = torch.arange(A, dtype=torch.int32)
+    private = [torch.arange(A + b * R, A + (b + 1) * R, dtype=torch.int32) for b in range(B)]
+    start = [50 + 10 * b for b in range(B)]
+    in_place = torch.cat([torch.cat([private[b][:start[b]], shared, private[b][start[b]:]]) for b in range(B)]).to(device)
+    shared_first = torch.cat([torch.cat([shared, private[b]]) for b in range(B)]).to(device)
+    cu_q = torch.arange(0, (B + 1) * q_per, q_per, dtype=torch.int32, device=device)
+    cu_k = torch.arange(0, (B + 1) * (A + R), A + R, dtype=torch.int32, device=device)
+    shifts = torch.tensor(start, dtype=torch.int32, device=device)
+    shared_lens = torch.full((B,), A, dtype=torch.int32, device=device)
+    flops = 4 * H * D * B * q_per * (A + R)
+    modes = []
+    for name, call in (
+            ("plain", lambda: ops.acache_attention(Q, K, V, cu_q, cu_k, in_place)),
+            ("key_side", lambda: ops.acache_attention(Q, K, V, cu_q, cu_k, in_place, None, A, None, shifts, cos, sin)),
+            ("query_side", lambda: ops.acache_attention(Q, K, V, cu_q, cu_k, shared_first, None, A, shared_lens, shifts,
+                                                        cos, sin))):
+        for _ in range(3):
+            call()
+        ms = _event_times_ms(call, steps, torch)[0]
+        modes.append({"mode": name, "us": round(ms * 1e3, 1), "TFLOPs": round(flops / ms / 1e9, 0)})
+    print(json.dumps({"attention_shape_sweep": rows, "relocation_modes": modes}))
 
 
 def kernel_sweep(torch, device, ops, steps):
