@@ -387,7 +387,7 @@ __global__ __launch_bounds__(256, RAGGED ? 1 : 2) void varlen_attn_kernel(AttnPa
 // One query tile of one (request, head): the NW waves (4 in every instantiation; the tile geometry below is
 // written in terms of NW so that it stays in one place) take WQ = 16 * NQ16 query rows each, starting at row
 // q_tile0 of the request, and stream the request's key tiles [t_begin, t_end) through the LDS ring.
-template <int DTYPE, int D, int NQ16, int MODE, int NW = 4>
+template <int DTYPE, int D, int NQ16, int MODE, int NW = 4, bool SMALL = false>
 __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0, char *lds_v0, char *lds_k1,
                                               char *lds_v1, float *lds_rope, int b, int q_begin, int q_len, int q_tile0,
                                               int head, int kvh, int t_begin, int t_end) {
@@ -468,33 +468,43 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   // ---- DMA bookkeeping: this lane's row and chunk inside each of its NI instructions
   const int dma_row0 = wave * WAVE_ROWS + lane / CH;   // + i*RPI
   const int dma_chunk = lane % CH;
-  const char *kc_base = p.k_cache + (int64_t)kvh * p.kv_head_bytes;
-  const char *vc_base = p.v_cache + (int64_t)kvh * p.kv_head_bytes;
+  // wave-uniform, and said so: the copies take them as scalar operands
+  const char *kc_base = uniform_ptr(p.k_cache + (int64_t)kvh * p.kv_head_bytes);
+  const char *vc_base = uniform_ptr(p.v_cache + (int64_t)kvh * p.kv_head_bytes);
 
   // slots of this lane's rows: even tiles in slot_a, odd tiles in slot_b (two named
   // register arrays, indexed statically).  load_slots only issues the loads; the
   // values are first touched by issue() one barrier later, so no wait for them is
   // ever placed in front of the MFMA work.
   int slot_a[NI], slot_b[NI];
+  const int32_t *const slot_lane = p.slot_map + kv_begin + dma_row0;   // + first key of the tile + i * RPI
   auto load_slots = [&](int t, int (&dst)[NI]) __attribute__((always_inline)) {
     const TileRange tr = tile_range_of(t < t_end ? t : t_end - 1, tiles_a, shared_len, kv_len, BN);
+    if (t < t_end && tr.n0 + BN <= tr.n_end) {
+      // full tile (a wave-uniform test): one address per lane, the row groups are immediate offsets
+      const int32_t *src = slot_lane + tr.n0;
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-      const int n = tr.n0 + dma_row0 + i * RPI;
-      // rows past the end of the range read index 0 (kv_len > 0, always readable);
-      // issue() ignores the value
-      dst[i] = p.slot_map[kv_begin + ((t < t_end && n < tr.n_end) ? n : 0)];
+      for (int i = 0; i < NI; ++i) dst[i] = src[i * RPI];
+    } else {
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int n = tr.n0 + dma_row0 + i * RPI;
+        // rows past the end of the range read index 0 (kv_len > 0, always readable);
+        // issue() ignores the value
+        dst[i] = p.slot_map[kv_begin + ((t < t_end && n < tr.n_end) ? n : 0)];
+      }
     }
   };
-  // Per-lane source addresses of row i of a tile, minus the slot term: base + swizzled chunk offset.
-  // One 64-bit multiply-add per row and tensor (slot * row pitch + this) is all the address math
-  // left in the loop.
-  const char *k_lane_src[NI], *v_lane_src[NI];
+  // Byte offset of this lane's (swizzled) chunk inside row i of a tile; the slot term is added per copy.  SMALL:
+  // the cache spans less than 4 GiB and slot numbers and the slot pitch fit 24 bits, so a copy's source is a
+  // wave-uniform base plus one 24-bit multiply-add (the 64-bit multiply-add of the general form runs at a
+  // quarter of that rate).
+  uint32_t k_lane_off[NI], v_lane_off_dma[NI];
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
     const int r = dma_row0 + i * RPI;
-    k_lane_src[i] = kc_base + ((dma_chunk ^ ((r / RW) % CH)) << 4);
-    v_lane_src[i] = vc_base + ((dma_chunk ^ (2 * ((r / RW) % (CH / 2)))) << 4);
+    k_lane_off[i] = (uint32_t)((dma_chunk ^ ((r / RW) % CH)) << 4);
+    v_lane_off_dma[i] = (uint32_t)((dma_chunk ^ (2 * ((r / RW) % (CH / 2)))) << 4);
   }
   const uint32_t slot_pitch = (uint32_t)p.kv_slot_bytes;
   const uint32_t slot_limit = p.num_slots > 0x7fffffffLL ? 0x7fffffffu : (uint32_t)p.num_slots;
@@ -513,9 +523,16 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   // this wave's rows inside a tile as a scalar byte offset (the lane's data lands 16 * lane behind the destination)
   const uint32_t wave_dst = __builtin_amdgcn_readfirstlane((uint32_t)(wave * WAVE_ROWS * ROW_BYTES));
   auto issue_rows = [&](int i, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
-    const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
-    lds_dma16_at(k_lane_src[i] + row_off, lds_offset_of(kbuf) + wave_dst + i * RPI * ROW_BYTES);
-    lds_dma16_at(v_lane_src[i] + row_off, lds_offset_of(vbuf) + wave_dst + i * RPI * ROW_BYTES);
+    const uint32_t dst = wave_dst + i * RPI * ROW_BYTES;
+    if (SMALL) {
+      const uint32_t row_off = __umul24((uint32_t)slots[i], slot_pitch);
+      lds_dma16_off(kc_base, row_off + k_lane_off[i], lds_offset_of(kbuf) + dst);
+      lds_dma16_off(vc_base, row_off + v_lane_off_dma[i], lds_offset_of(vbuf) + dst);
+    } else {
+      const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
+      lds_dma16_at(kc_base + (row_off + k_lane_off[i]), lds_offset_of(kbuf) + dst);
+      lds_dma16_at(vc_base + (row_off + v_lane_off_dma[i]), lds_offset_of(vbuf) + dst);
+    }
   };
   auto issue_slow = [&](int t, char *kbuf, char *vbuf, const int (&slots)[NI]) __attribute__((always_inline)) {
     const TileRange tr = tile_range_of(t, tiles_a, shared_len, kv_len, BN);
@@ -525,8 +542,8 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
       const int r = dma_row0 + i * RPI;
       const bool present = tr.n0 + r < tr.n_end && (uint32_t)slots[i] < slot_limit;
       const uint64_t row_off = (uint64_t)(uint32_t)slots[i] * slot_pitch;
-      const char *ksrc = present ? k_lane_src[i] + row_off : zero;
-      const char *vsrc = present ? v_lane_src[i] + row_off : zero;
+      const char *ksrc = present ? kc_base + (row_off + k_lane_off[i]) : zero;
+      const char *vsrc = present ? vc_base + (row_off + v_lane_off_dma[i]) : zero;
       lds_dma16_at(ksrc, lds_offset_of(kbuf) + wave_dst + i * RPI * ROW_BYTES);
       lds_dma16_at(vsrc, lds_offset_of(vbuf) + wave_dst + i * RPI * ROW_BYTES);
     }
@@ -559,6 +576,16 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   const int v_swz = ((v_row / RW) % (CH / 2));            // f_V(row)/2; rows differ by multiples of 16
   const int v_lane_off = v_row * ROW_BYTES + ((v_ib >> 1) << 4) + ((v_ib & 1) << 3);
   const float c = p.scale_log2e;
+  // LDS addresses of this lane's fragments inside the ring's first K tile: the tile (K0, V0, K1, V1 lie 16 KiB
+  // apart), the 16-key block and the slab are immediates of the read instructions
+  typedef __attribute__((address_space(3))) const char *LdsBytes;
+  LdsBytes k_frag[KS], v_frag[DT];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks)
+    k_frag[ks] = (LdsBytes)lds_k0 + (li * ROW_BYTES + (((4 * ks + lg) ^ k_swz) << 4));
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    v_frag[dt] = (LdsBytes)lds_k0 + (v_lane_off + (((dt ^ v_swz) & (CH / 2 - 1)) << 5));
 
   // MASKED = true: keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
   // stepped: the copies of the next tile (into nk / nv, slots nslots) ride along, one row group at
@@ -582,7 +609,9 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
       for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const vec16 kf = load16(kbuf + (16 * nt + li) * ROW_BYTES + (((4 * ks + lg) ^ k_swz) << 4));
+          typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+          const u32x4 kraw = *(__attribute__((address_space(3))) const u32x4 *)(k_frag[ks] + ((kbuf - lds_k0) + 16 * nt * ROW_BYTES));
+          const vec16 kf{{kraw.x, kraw.y, kraw.z, kraw.w}};
 #pragma unroll
           for (int qt = 0; qt < NQ16; ++qt)
             s_acc[qt][nt] = M::run(kf, qq[qt][ks], s_acc[qt][nt]);
@@ -614,8 +643,7 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     auto pv_slab = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
-        const int col = (((dt ^ v_swz) & (CH / 2 - 1)) << 5);  // swizzled 32-byte column block of d tile dt
-        const char *src = vbuf + v_lane_off + 32 * s * ROW_BYTES + col;
+        const LdsBytes src = v_frag[dt] + ((vbuf - lds_k0) + 32 * s * ROW_BYTES);
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)src);
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
             (s16x4 __attribute__((address_space(3))) *)(src + 16 * ROW_BYTES));
@@ -814,7 +842,7 @@ __device__ __forceinline__ int sk_key_tiles(const AttnParams &p, int b, int kv_l
 
 // One workgroup per unit, units dealt whole: blocks are handed out in index order, which with the
 // longest-request-first tile order of locate_query_tile_lpt is longest-processing-time-first list scheduling.
-template <int DTYPE, int D, int MODE, int NW = 4>
+template <int DTYPE, int D, int MODE, bool SMALL, int NW = 4>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_kernel(AttnParams p) {
   constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = 64 * D * 2;
@@ -842,10 +870,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
   const int q_tile0 = tile * BM;
   const int kt = sk_key_tiles<MODE>(p, b, p.cu_k[b + 1] - p.cu_k[b]);
   if (q_len - q_tile0 <= BM / 2)
-    attn_dma_part<DTYPE, D, 1, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
+    attn_dma_part<DTYPE, D, 1, MODE, NW, SMALL>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
                                          0, kt);
   else
-    attn_dma_part<DTYPE, D, 2, MODE, NW>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
+    attn_dma_part<DTYPE, D, 2, MODE, NW, SMALL>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
                                          0, kt);
 }
 
@@ -856,12 +884,19 @@ static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStrea
   p.num_tiles = (int32_t)((total_q + 127) / 128) + p.B;
   const int64_t blocks = attn_grid_blocks(p);
   if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
-  if (mode == MODE_PLAIN)
-    hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_PLAIN>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
-  else if (mode == MODE_KEY_SIDE)
-    hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_KEY_SIDE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, MODE_QUERY_SIDE>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  // 32-bit copy offsets when the whole cache lies within 4 GiB of a head's base and the factors fit 24 bits
+  const bool small = p.num_slots < (1 << 24) && p.kv_slot_bytes > 0 && p.kv_slot_bytes < (1 << 24) &&
+                     p.num_slots * p.kv_slot_bytes + 4096 <= 0xffffffffLL;
+  const dim3 grid((unsigned)blocks), block(256);
+#define ACACHE_UNIT(M)                                                                              \
+  if (mode == M) {                                                                                  \
+    if (small) hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, M, true>), grid, block, 0, stream, p); \
+    else hipLaunchKernelGGL((varlen_attn_unit_kernel<DTYPE, D, M, false>), grid, block, 0, stream, p);      \
+  }
+  ACACHE_UNIT(MODE_PLAIN)
+  ACACHE_UNIT(MODE_KEY_SIDE)
+  ACACHE_UNIT(MODE_QUERY_SIDE)
+#undef ACACHE_UNIT
   return launch_status("varlen_attn_unit_kernel");
 }
 

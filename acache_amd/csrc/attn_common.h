@@ -185,6 +185,18 @@ __device__ __forceinline__ void lds_dma16_at(const char *src, uint32_t lds_offse
   asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "{m0}"(lds_offset) : "memory");
 }
 
+// A pointer every lane holds the same value of, moved to scalar registers.
+__device__ __forceinline__ const char *uniform_ptr(const char *p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return reinterpret_cast<const char *>(((uint64_t)hi << 32) | lo);
+}
+// The copy with the source given as a wave-uniform base plus a 32-bit byte offset per lane.
+__device__ __forceinline__ void lds_dma16_off(const char *base, uint32_t offset, uint32_t lds_offset) {
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "{m0}"(lds_offset) : "memory");
+}
+
 // Online-softmax update of one key tile, in two steps shared by both attention kernels so that
 // they round identically (key-side relocation must reproduce a materialised copy bit for bit).
 //

@@ -356,6 +356,32 @@ def test_anchor_recompute_config_full_size_against_library_attention_on_device(d
     assert (got_p.float() - got.float()).abs().max().item() <= 4e-3
 
 
+def test_wide_slot_pitch_takes_the_64_bit_copy_addresses(device):
+    """The copies address a compact cache (less than 4 GiB, slot pitch below 2^24 bytes) with 32-bit offsets from a
+    scalar base and anything else with 64-bit addresses.  A cache whose slots lie 16 MiB apart takes the second
+    form; its result must be the same bits as that of the same rows in a compact cache."""
+    torch.manual_seed(5)
+    H = Hkv = 8
+    D, S = 128, 24
+    pitch = 1 << 23   # elements: 16 MiB per slot
+    q_lens, kv_lens = [70, 33], [S, S - 5]
+    cu_q = torch.tensor([0, 70, 103], dtype=torch.int32, device=device)
+    cu_k = torch.tensor([0, S, 2 * S - 5], dtype=torch.int32, device=device)
+    slots = torch.cat([torch.randperm(S), torch.randperm(S)[:S - 5]]).to(torch.int32).to(device)
+    q = (torch.randn(103, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+    kc = (torch.randn(S, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+    vc = torch.randn(S, Hkv, D, device=device).to(torch.bfloat16)
+    wide_k = torch.zeros(S * pitch, dtype=torch.bfloat16, device=device).as_strided((S, Hkv, D), (pitch, D, 1))
+    wide_v = torch.zeros(S * pitch, dtype=torch.bfloat16, device=device).as_strided((S, Hkv, D), (pitch, D, 1))
+    wide_k.copy_(kc)
+    wide_v.copy_(vc)
+    compact = ops.acache_attention(q, kc, vc, cu_q, cu_k, slots)
+    wide = ops.acache_attention(q, wide_k, wide_v, cu_q, cu_k, slots)
+    assert torch.equal(compact, wide)
+    want = O.acache_attention(q.cpu(), kc.cpu(), vc.cpu(), cu_q.cpu(), cu_k.cpu(), slots.cpu())
+    _close(compact, want)
+
+
 def test_block_table_variants(device):
     """baseline_ragged_attention / baseline_decode_attention geometry of tests/test_attention_kernels.py:371-476,
     checked against dense attention over the un-paged K/V."""
