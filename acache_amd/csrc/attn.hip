@@ -15,21 +15,24 @@
 //   MFMA row block (V^T rows of ones).
 //
 // Two kernels:
-//   varlen_attn_dma_kernel (plain and query-side relocation): K/V rows are copied
-//     global -> LDS directly through the slot map into a two-deep ring, swizzled by
-//     permuting the global side of the copy; V stays row-major and is read with
-//     the LDS transpose read.
-//   varlen_attn_kernel (key-side relocation): rows are staged through registers,
-//     re-rotated there, and V is transposed on the way into LDS.
-// Both share the softmax steps below, so they round identically.  HBM traffic per
-// call: K and V rows once per (request, kv head) when query tiles of one head share
-// an L2 (block indices are mapped so that they land on the same XCD), Q once, O once.
+//   varlen_attn_unit_kernel (head_dim 64 and 128, all three relocation modes): K/V rows are copied
+//     global -> LDS directly through the slot map into a two-deep ring, swizzled by permuting the
+//     global side of the copy; V stays row-major and is read with the LDS transpose read.  Queries are
+//     multiplied by scale * log2 e when their fragments are loaded and the score accumulators start
+//     at minus the softmax reference, so a probability is exp2 of its accumulator as it stands.
+//     Key-side relocation re-rotates the shared rows of a tile in LDS once it has landed.
+//   varlen_attn_kernel (any other head_dim): rows are staged through registers, re-rotated there in
+//     key-side mode, and V is transposed on the way into LDS; scores are scaled in the softmax.
+// Within a kernel all modes share the softmax steps, so key-side relocation rounds exactly like
+// attention over a materialised copy.  HBM traffic per call: K and V rows once per (request, kv head)
+// when query tiles of one head share an L2 (block indices are mapped so that they land on the same
+// XCD), Q once, O once.
 #include <stdlib.h>
 #include "attn_common.h"
 
 namespace acache {
 
-// Register-staged kernel: key-side relocation at head_dim 64 / 128, and every mode at any other head_dim.
+// Register-staged kernel: every mode at a head_dim other than 64 / 128.
 //
 // RAGGED = true is the any-head_dim variant: D is then the padded width (a multiple of 32) and the real
 // head_dim (a multiple of 16, at most D) comes in p.head_dim.  Rows are laid out in LDS at their real
@@ -461,6 +464,15 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
         for (int ks = 0; ks < KS / 2; ++ks)
           rotate_pair<DTYPE, D>(qf[qt][ks], qf[qt][ks + KS / 2], cr, sr, 32 * ks + 8 * lg, -1.0f);
       }
+      // queries are scored as q * scale * log2 e (rounded to the cache type once more), so the scores come out
+      // of the matrix core in the log2 units the softmax works in
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        float f[8];
+        Elem<DTYPE>::unpack(qf[qt][ks], f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qf[qt][ks].w[j] = M::pack2(f[2 * j] * p.scale_log2e, f[2 * j + 1] * p.scale_log2e);
+      }
     }
   };
   load_q(MODE == MODE_QUERY_SIDE && t_begin < tiles_a);
@@ -557,10 +569,14 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     }
   };
 
+  // m_run: reference point of the running sums in log2 units; neg_m: minus the value the score accumulators
+  // start at (the reference, or 0 in front of the first tile), replicated as an accumulator operand
   float m_run[NQ16];
   f32x4 o_acc[NQ16][DT], l_acc[NQ16];
+  f32x4 neg_m[NQ16];
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
+    neg_m[qt] = f32x4{0, 0, 0, 0};
     m_run[qt] = -INFINITY;
     l_acc[qt] = f32x4{0, 0, 0, 0};
 #pragma unroll
@@ -575,7 +591,6 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   const int v_row = 4 * lg + v_j;                         // + 32*s (+16 for the second half)
   const int v_swz = ((v_row / RW) % (CH / 2));            // f_V(row)/2; rows differ by multiples of 16
   const int v_lane_off = v_row * ROW_BYTES + ((v_ib >> 1) << 4) + ((v_ib & 1) << 3);
-  const float c = p.scale_log2e;
   // LDS addresses of this lane's fragments inside the ring's first K tile: the tile (K0, V0, K1, V1 lie 16 KiB
   // apart), the 16-key block and the slab are immediates of the read instructions
   typedef __attribute__((address_space(3))) const char *LdsBytes;
@@ -603,7 +618,7 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] = f32x4{0, 0, 0, 0};
+      for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] = neg_m[qt];  // the accumulators start at minus the reference
     auto scores = [&](const vec16 (&qq)[NQ16][KS]) __attribute__((always_inline)) {
 #pragma unroll
       for (int nt = 0; nt < NT; ++nt) {
@@ -633,7 +648,7 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     __builtin_amdgcn_s_setprio(0);
 
     copy_point(1);
-    softmax_reference<NQ16, NQ16, NT, DT, MASKED>(s_acc, m_run, l_acc, o_acc, c, n_valid, lg);
+    softmax_reference_prescaled<NQ16, NQ16, NT, DT, MASKED>(s_acc, m_run, neg_m, l_acc, o_acc, n_valid, lg);
     copy_point(2);
 
     // O^T += V^T P^T, one 32-key slab at a time, so that the exponentials of the second slab
@@ -654,11 +669,11 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
           o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
       }
     };
-    softmax_probs_slab<M, 0, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
+    softmax_probs_slab_prescaled<M, 0, NQ16>(s_acc, l_acc, pf, ones);
     copy_point(3);
     __builtin_amdgcn_s_setprio(1);
     pv_slab(0);
-    softmax_probs_slab<M, 1, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
+    softmax_probs_slab_prescaled<M, 1, NQ16>(s_acc, l_acc, pf, ones);
     pv_slab(1);
     // Issue order: V fragments two d-tiles ahead of their use.
     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -709,7 +724,9 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
       char *row = kbuf + rot_row * ROW_BYTES;
       const int f = (rot_row / RW) % CH;
       auto rotate_with = [&](const float *cr, const float *sr, float sign) __attribute__((always_inline)) {
-#pragma unroll
+        // a real loop: unrolled, the loads of both chunk pairs are hoisted to the front and the kernel spills
+        // (21 registers, 12 % slower in key-side mode)
+#pragma nounroll
         for (int k = 0; k < PER_THREAD; ++k) {
           const int c = (tid % (PAIRS / PER_THREAD)) * PER_THREAD + k;
           char *lo_p = row + ((c ^ f) << 4), *hi_p = row + (((c + PAIRS) ^ f) << 4);
