@@ -330,7 +330,7 @@ int acache_build_slot_layout(
  *   fp32 accumulation, probabilities rounded to `dtype` before the PV product,
  *   output rounded to `dtype`.  At head_dim 64 / 128 the scale is applied to the
  *   query (q * scale * log2 e rounded to `dtype`, exp2 of the fp32 product) where
- *   the reference scales the fp32 product (line 453): one more rounding of q, within
+ *   the reference scales the fp32 product (lines 439, 460, 499): one more rounding of q, within
  *   the 2e-2 absolute bound on outputs the parity tests hold this call to.
  *
  * Relocation modes (selected exactly as the reference wrapper does,
