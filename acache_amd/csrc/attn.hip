@@ -390,10 +390,10 @@ __global__ __launch_bounds__(256, RAGGED ? 1 : 2) void varlen_attn_kernel(AttnPa
 // One query tile of one (request, head): the NW waves (4 in every instantiation; the tile geometry below is
 // written in terms of NW so that it stays in one place) take WQ = 16 * NQ16 query rows each, starting at row
 // q_tile0 of the request, and stream the request's key tiles [t_begin, t_end) through the LDS ring.
-template <int DTYPE, int D, int NQ16, int MODE, int NW = 4, bool SMALL = false>
+template <int DTYPE, int D, int NQ16, int MODE, int NW = 4, bool SMALL = false, int KSPLIT = 1>
 __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0, char *lds_v0, char *lds_k1,
                                               char *lds_v1, float *lds_rope, int b, int q_begin, int q_len, int q_tile0,
-                                              int head, int kvh, int t_begin, int t_end) {
+                                              int head, int kvh, int kv_begin, int kv_len, int t_begin, int t_end) {
   constexpr int BN = 64;
   constexpr int WQ = 16 * NQ16;
   constexpr int KS = D / 32;
@@ -408,6 +408,15 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   constexpr int THREADS = 64 * NW;
   constexpr int NI = WAVE_ROWS / RPI;         // DMA instructions per wave, tile and tensor: 4 or 2
   constexpr int TILE_BYTES = BN * ROW_BYTES;
+  // KSPLIT = 2 (query tiles of at most half the rows): waves 2g and 2g + 1 hold the same WQ query rows and take
+  // the first and the second 32 keys of every tile; their partial (reference, denominator, O) triples are merged
+  // through LDS behind the key loop.  Every wave still copies its 16 rows of each tile.
+  static_assert(KSPLIT == 1 || (KSPLIT == 2 && NW == 4), "key split: one or two waves per query row group");
+  // Short query tiles have too little work per key tile to hide a copy issued in the middle of it: all copies of
+  // the next tile go out right behind the barrier.
+  constexpr bool COPY_EARLY = KSPLIT == 2;
+  constexpr int NTL = NT / KSPLIT;            // 16-key blocks of a tile that a wave scores
+  constexpr int NSL = NS / KSPLIT;            // 32-key slabs of a tile that a wave multiplies into O
   using M = Mma<DTYPE>;
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   // An opaque zero keeps the compiler from computing the lane-derived address constants below ahead of the
@@ -418,15 +427,14 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   const int tid = threadIdx.x + opaque_zero;
   const int lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, lg = lane >> 4;
-  const int kv_begin = p.cu_k[b];
-  const int kv_len = p.cu_k[b + 1] - kv_begin;
-  const int q_wave0 = q_tile0 + wave * WQ;
+  const int kp = KSPLIT == 1 ? 0 : __builtin_amdgcn_readfirstlane(wave % KSPLIT);  // which part of a tile's keys
+  const int q_wave0 = q_tile0 + (wave / KSPLIT) * WQ;
   int nq_valid = (q_len - q_wave0 + 15) / 16;
   nq_valid = nq_valid < 0 ? 0 : (nq_valid > NQ16 ? NQ16 : nq_valid);
   char *out_base = p.out + (int64_t)q_begin * p.o_token_bytes + (int64_t)head * p.o_head_bytes;
 
   if (kv_len <= 0) {
-    for (int r = tid / CH; r < NW * WQ; r += THREADS / CH) {
+    for (int r = tid / CH; r < NW / KSPLIT * WQ; r += THREADS / CH) {
       const int qr = q_tile0 + r;
       if (qr < q_len) store16(out_base + (int64_t)qr * p.o_token_bytes + (tid % CH) * 16, vec16{{0, 0, 0, 0}});
     }
@@ -597,10 +605,10 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   LdsBytes k_frag[KS], v_frag[DT];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
-    k_frag[ks] = (LdsBytes)lds_k0 + (li * ROW_BYTES + (((4 * ks + lg) ^ k_swz) << 4));
+    k_frag[ks] = (LdsBytes)lds_k0 + (li * ROW_BYTES + (((4 * ks + lg) ^ k_swz) << 4) + kp * (BN / KSPLIT) * ROW_BYTES);
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
-    v_frag[dt] = (LdsBytes)lds_k0 + (v_lane_off + (((dt ^ v_swz) & (CH / 2 - 1)) << 5));
+    v_frag[dt] = (LdsBytes)lds_k0 + (v_lane_off + (((dt ^ v_swz) & (CH / 2 - 1)) << 5) + kp * (BN / KSPLIT) * ROW_BYTES);
 
   // MASKED = true: keys at tile rows >= n_valid are absent (last tile of a range) and get score -inf.
   // stepped: the copies of the next tile (into nk / nv, slots nslots) ride along, one row group at
@@ -611,17 +619,17 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
       if (stepped) {
 #pragma unroll
         for (int i = 0; i < NI; ++i)
-          if (i * 4 / NI == point) issue_rows(i, nk, nv, nslots);
+          if ((COPY_EARLY ? 0 : i * 4 / NI) == point) issue_rows(i, nk, nv, nslots);
       }
     };
-    f32x4 s_acc[NQ16][NT];
+    f32x4 s_acc[NQ16][NTL];
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt)
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] = neg_m[qt];  // the accumulators start at minus the reference
+      for (int nt = 0; nt < NTL; ++nt) s_acc[qt][nt] = neg_m[qt];  // the accumulators start at minus the reference
     auto scores = [&](const vec16 (&qq)[NQ16][KS]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int nt = 0; nt < NT; ++nt) {
+      for (int nt = 0; nt < NTL; ++nt) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -640,7 +648,7 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     // instructions) ahead of their use, so LDS latency hides behind the matrix core.
     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-    for (int i = 0; i < (NT * KS - 4) / 2; ++i) {
+    for (int i = 0; i < (NTL * KS - 4) / 2; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 2 * NQ16, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
@@ -648,13 +656,14 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     __builtin_amdgcn_s_setprio(0);
 
     copy_point(1);
-    softmax_reference_prescaled<NQ16, NQ16, NT, DT, MASKED>(s_acc, m_run, neg_m, l_acc, o_acc, n_valid, lg);
+    softmax_reference_prescaled<NQ16, NQ16, NTL, DT, MASKED>(s_acc, m_run, neg_m, l_acc, o_acc,
+                                                             n_valid - kp * (BN / KSPLIT), lg);
     copy_point(2);
 
     // O^T += V^T P^T, one 32-key slab at a time, so that the exponentials of the second slab
     // have the matrix-core work of the first to hide behind.
     static_assert(NS == 2, "two 32-key slabs per tile");
-    vec16 pf[NQ16][NS];
+    vec16 pf[NQ16][NSL];
     auto pv_slab = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -672,17 +681,19 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     softmax_probs_slab_prescaled<M, 0, NQ16>(s_acc, l_acc, pf, ones);
     copy_point(3);
     __builtin_amdgcn_s_setprio(1);
-    pv_slab(0);
-    softmax_probs_slab_prescaled<M, 1, NQ16>(s_acc, l_acc, pf, ones);
-    pv_slab(1);
+    pv_slab(0);  // with a key split this is the wave's own slab: its offset is part of v_frag
+    if constexpr (NSL == 2) {
+      softmax_probs_slab_prescaled<M, 1, NQ16>(s_acc, l_acc, pf, ones);
+      pv_slab(1);
+    }
     // Issue order: V fragments two d-tiles ahead of their use.
     __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-    for (int i = 0; i < 2 * DT - 2; ++i) {
+    for (int i = 0; i < NSL * DT - 2; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, NQ16, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, 3 * NQ16, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, (NSL + 1) * NQ16, 0);
     __builtin_amdgcn_s_setprio(0);
   };
 
@@ -811,6 +822,38 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
   }
   __syncthreads();  // every wave is done reading the K/V ring
 
+  // ---- key split: the odd wave of a pair hands its partial state to the even one ---------------
+  // Both waves hold the same queries in the same lanes, so the merge is lane-local.  The odd wave parks O (fp32,
+  // in register order: exactly one ring buffer) in its own output-staging buffer and (reference, denominator)
+  // at the end of its partner's; a wave that never saw a key (requests of at most 32 keys) reports -inf.
+  if constexpr (KSPLIT == 2) {
+    static_assert(NQ16 * DT * 64 * 16 <= TILE_BYTES, "a wave's partial O must fit one ring buffer");
+    f32x4 *xo = reinterpret_cast<f32x4 *>(lds_k0 + (wave | 1) * TILE_BYTES);
+    // (the last KiB of the even wave's buffer: its output staging below uses less than the first 9 KiB)
+    static_assert(WQ * (ROW_BYTES + 16) + NQ16 * 2 * 64 * 4 <= TILE_BYTES, "room for the exchanged statistics");
+    float *xml = reinterpret_cast<float *>(lds_k0 + ((wave & ~1) + 1) * TILE_BYTES - NQ16 * 2 * 64 * 4);
+    if (kp == 1) {
+#pragma unroll
+      for (int qt = 0; qt < NQ16; ++qt) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) xo[(qt * DT + dt) * 64 + lane] = o_acc[qt][dt];
+        xml[(2 * qt) * 64 + lane] = kv_len > BN / KSPLIT ? m_run[qt] : -INFINITY;
+        xml[(2 * qt + 1) * 64 + lane] = l_acc[qt][0];
+      }
+    }
+    __syncthreads();
+    if (kp == 1) return;
+#pragma unroll
+    for (int qt = 0; qt < NQ16; ++qt) {
+      const float m1 = xml[(2 * qt) * 64 + lane], l1 = xml[(2 * qt + 1) * 64 + lane];
+      const float ms = fmaxf(m_run[qt], m1);
+      const float a0 = __builtin_amdgcn_exp2f(m_run[qt] - ms), a1 = __builtin_amdgcn_exp2f(m1 - ms);
+      l_acc[qt][0] = l_acc[qt][0] * a0 + l1 * a1;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] = o_acc[qt][dt] * a0 + xo[(qt * DT + dt) * 64 + lane] * a1;
+    }
+  }
+
   // ---- epilogue: normalise, transpose through LDS, store whole 16-byte chunks ------------------
   // Lane layout of O^T (query li, features 16*dt + 4*lg .. +4) would give 8-byte stores scattered
   // over 16 rows; staging the wave's WQ x D tile in LDS (one 16 KiB ring buffer per wave, rows padded
@@ -876,22 +919,30 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
   if (!block_to_tile_head(p, tile, kvh, hg)) return;
   const int group = p.H / p.H_kv;
   const int head = kvh * group + hg;
-  int b = 0, q_begin = 0, q_len = 0;
+  int b = 0, q_begin = 0, q_len = 0, kv_begin = 0, kv_len = 0;
   {
     int tile_in_request = 0;
-    const bool found = p.B <= 64 ? locate_query_tile_lpt(p.cu_q, p.cu_k, p.B, BM, tile, b, q_begin, q_len, tile_in_request)
-                                 : locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request);
-    if (!found) return;
+    if (p.B <= 64) {
+      if (!locate_query_tile_lpt(p.cu_q, p.cu_k, p.B, BM, tile, b, q_begin, q_len, tile_in_request, kv_begin, kv_len)) return;
+    } else {
+      if (!locate_query_tile(p.cu_q, p.B, BM, tile, b, q_begin, q_len, tile_in_request)) return;
+      kv_begin = p.cu_k[b];
+      kv_len = p.cu_k[b + 1] - kv_begin;
+    }
     tile = tile_in_request;
   }
   const int q_tile0 = tile * BM;
-  const int kt = sk_key_tiles<MODE>(p, b, p.cu_k[b + 1] - p.cu_k[b]);
-  if (q_len - q_tile0 <= BM / 2)
-    attn_dma_part<DTYPE, D, 1, MODE, NW, SMALL>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
-                                         0, kt);
+  const int kt = sk_key_tiles<MODE>(p, b, kv_len);
+  // tiles with at most 64 (32) live rows: two waves per 32 (16) rows, each on half of every tile's keys
+  if (q_len - q_tile0 <= BM / 4)
+    attn_dma_part<DTYPE, D, 1, MODE, NW, SMALL, 2>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len,
+                                                   q_tile0, head, kvh, kv_begin, kv_len, 0, kt);
+  else if (q_len - q_tile0 <= BM / 2)
+    attn_dma_part<DTYPE, D, 2, MODE, NW, SMALL, 2>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len,
+                                                   q_tile0, head, kvh, kv_begin, kv_len, 0, kt);
   else
-    attn_dma_part<DTYPE, D, 2, MODE, NW, SMALL>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len, q_tile0, head, kvh,
-                                         0, kt);
+    attn_dma_part<DTYPE, D, 2, MODE, NW, SMALL>(p, lds_k0, lds_v0, lds_k1, lds_v1, lds_rope, b, q_begin, q_len,
+                                                q_tile0, head, kvh, kv_begin, kv_len, 0, kt);
 }
 
 template <int DTYPE, int D, int NQ16>

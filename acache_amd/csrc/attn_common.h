@@ -81,11 +81,15 @@ __device__ __forceinline__ bool locate_query_tile(const int32_t *cu_q, int B, in
 // list scheduling: the short blocks fill the gaps at the end instead of the long ones sticking out.
 __device__ __forceinline__ bool locate_query_tile_lpt(const int32_t *cu_q, const int32_t *cu_k, int B, int BM,
                                                       int rank, int &b_out, int &q_begin, int &q_len,
-                                                      int &tile_in_request) {
+                                                      int &tile_in_request, int &kv_begin, int &kv_len) {
   const int lane = threadIdx.x & 63;
-  const int lo = lane < B ? cu_q[lane] : 0;
-  const int len = lane < B ? cu_q[lane + 1] - lo : 0;
-  const int kv = lane < B ? cu_k[lane + 1] - cu_k[lane] : 0;
+  // four unconditional loads at a clamped index: one memory round trip (loads under a lane mask end up in
+  // separate blocks, each with its own wait)
+  const int l = lane < B ? lane : B - 1;
+  const int q0 = cu_q[l], q1 = cu_q[l + 1], k0 = cu_k[l], k1 = cu_k[l + 1];
+  const int lo = q0;
+  const int len = lane < B ? q1 - q0 : 0;
+  const int kv = lane < B ? k1 - k0 : 0;
   const int tiles = len > 0 ? (len + BM - 1) / BM : 0;
   int before = 0;  // query tiles of the requests sorted in front of this lane's request
   for (int j = 0; j < B; ++j) {
@@ -97,9 +101,11 @@ __device__ __forceinline__ bool locate_query_tile_lpt(const int32_t *cu_q, const
   if (hit == 0) return false;
   const int src = __builtin_ctzll(hit);
   b_out = src;
-  q_begin = __shfl(lo, src);
-  q_len = __shfl(len, src);
-  tile_in_request = rank - __shfl(before, src);
+  q_begin = __builtin_amdgcn_readlane(lo, src);
+  q_len = __builtin_amdgcn_readlane(len, src);
+  tile_in_request = rank - __builtin_amdgcn_readlane(before, src);
+  kv_begin = __builtin_amdgcn_readlane(k0, src);
+  kv_len = __builtin_amdgcn_readlane(kv, src);
   return true;
 }
 
