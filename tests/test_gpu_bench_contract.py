@@ -47,5 +47,10 @@ def test_default_line_has_the_contract_keys(device):
         assert leg["cpu_baseline"]["value"] > 0 and leg["cpu_baseline"]["sample"], name
     assert d["relocate_fp32"]["affix_only"]["rows"] == 512 and d["relocate_fp32"]["whole_buffer"]["rows"] == 896
     assert d["anchor_select_scatter"]["topk"]["us_per_launch"] > 0
-    modes = [r["mode"] for r in d["engine"]["results"]]
-    assert modes == ["full_recompute", "acache_0.2"] and d["engine"]["speedup_vs_full_recompute"] > 0
+    # the whole anchor-ratio sweep of the engine configuration, against full affix recompute; headline = ratio 0.2
+    rows = d["engine"]["results"]
+    assert [r["mode"] for r in rows] == ["full_recompute", "acache_0.0", "acache_0.1", "acache_0.2", "acache_0.3",
+                                         "acache_0.5", "acache_1.0"]
+    assert all(r["tokens_per_s"] > 0 and r["speedup_vs_full_recompute"] > 0 for r in rows)
+    assert d["engine"]["value"] == rows[3]["tokens_per_s"] and d["engine"]["speedup_vs_full_recompute"] > 0
+    assert "sets used in turn" in d["anchor_select_scatter"]["config"]["workload"]
