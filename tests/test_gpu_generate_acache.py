@@ -47,7 +47,8 @@ def _fixture(device, as_checkpoint_object=False):
 def test_importance_matches_the_reference_fixture(device, as_checkpoint_object):
     """compute_attention_importance_cross_affix against the values the reference returned for prefix, infix and
     suffix placement.  The reference ran in fp32, the engine in bf16 with the relocation on the query side:
-    measured difference 0.044 absolute / 4.6 % relative at most; bound 0.1 / 8 %.  The anchors chosen from the two
+    measured difference 0.044 absolute / 4.6 % relative at most; bound 0.06 / 6 %, and the total weight (mask rows x
+    heads x layers, which a per-layer weighting slip would change) within 0.5 %.  The anchors chosen from the two
     importance vectors must be the same tokens."""
     cases, model = _fixture(device, as_checkpoint_object)
     for c in cases:
@@ -57,7 +58,8 @@ def test_importance_matches_the_reference_fixture(device, as_checkpoint_object):
                                                          affix_start=kw["affix_start"]).cpu()
         want = c["importance"]
         assert got.shape == want.shape
-        torch.testing.assert_close(got, want, rtol=8e-2, atol=1e-1, msg=lambda m: f"{c['name']}: {m}")
+        torch.testing.assert_close(got, want, rtol=6e-2, atol=6e-2, msg=lambda m: f"{c['name']}: {m}")
+        assert abs(got.sum().item() - want.sum().item()) <= 5e-3 * want.sum().item(), c["name"]
         k = G.ceil_to_int(kw["anchor_ratio"] * want.shape[1])
         assert (G.select_anchor_tokens(got.to(device), k, "top").tolist()
                 == G.select_anchor_tokens(want.to(device), k, "top").tolist()), c["name"]
