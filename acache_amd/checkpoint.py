@@ -3,7 +3,8 @@
 The reference's entry points are handed the checkpoint's own model class (llada/eval_ACache.py:100-107, 189 and
 dream/eval_ACache.py for the HF path; nano-vdllm's ``ModelRunner(model, config)``, model_runner.py:15-19, for the
 engine).  Those classes carry their own attention; the engine needs this package's blocks.  ``engine_model_for``
-bridges the two without copying weights."""
+bridges the two; ``llada.adopt_state`` says which tensors are shared with the checkpoint object and which are
+merged copies."""
 from __future__ import annotations
 
 import weakref

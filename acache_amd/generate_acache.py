@@ -11,8 +11,9 @@ non-affix tokens recomputed at every block boundary, block-only refinement in be
 the paged engine of this package (``ModelRunner`` + HIP kernels).  Consequences for callers:
 
 * ``model`` is the checkpoint model object the reference's caller passes (llada/eval_ACache.py:100-107, 189):
-  the engine model is built around its parameter tensors on first use (no second copy of the weights; settings
-  the engine's decoder stack does not implement raise ``TypeError``).  An engine model
+  the engine model is built around its parameter tensors on first use (the q/k/v and gate/up projections become
+  merged copies, everything else is shared: ``llada.adopt_state``; settings the engine's decoder stack does not
+  implement raise ``TypeError``).  An engine model
   (``acache_amd.llada.LLaDAModelLM``) or a ready ``ModelRunner`` is taken as it is;
 * ``precomputed_affix_cache`` is optional.  ``None``: the affix is encoded once into the shared
   slots.  A per-layer tuple of ``(k, v)`` with the HF layout ``[1, H_kv, A, D]`` and PRE-RoPE keys

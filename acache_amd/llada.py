@@ -132,6 +132,12 @@ class LLaDABlock(nn.Module):
             cached = self._fused[name] = (w, b)
         return cached
 
+    def fuse_projections(self):
+        """Build the merged q/k/v and gate/up weights now rather than on the first forward, so that whoever sizes
+        the KV cache from free device memory afterwards already sees them."""
+        self._fuse("qkv", (self.q_proj, self.k_proj, self.v_proj))
+        self._fuse("gate_up", (self.ff_proj, self.up_proj))
+
     @staticmethod
     def _hooked(*linears):
         # a projection somebody observes (forward hooks) keeps its own forward call
@@ -203,7 +209,8 @@ class LLaDAModel(nn.Module):
     def forward(self, input_ids, position_ids=None, compute_logits=True, logits_keep_indices=None):
         if position_ids is None:
             position_ids = torch.arange(input_ids.shape[-1], device=input_ids.device).expand_as(input_ids)
-        max_pos = self.config.max_sequence_length
+        # rows of the rotary table: the configured length, or more when the runner serves a longer request
+        max_pos = max(self.config.max_sequence_length, int(getattr(self, "rope_positions", 0)))
         x = self.transformer["wte"](input_ids)
         blocks = self.transformer["blocks"]
         ln_f = self.transformer["ln_f"]
@@ -253,7 +260,8 @@ class LLaDAModelLM(nn.Module):
 # (llada/eval_ACache.py:100-107 loads llada/model/modeling_llada.py:LLaDAModelLM in bf16 and passes it to
 # generate_with_anchor_attention, :189).  That class attends over dense [B, H, L, D] caches inside its own
 # forward and cannot run on the paged engine, but its parameters can: this module's blocks use the same
-# parameter names, so the engine model is built around the checkpoint's tensors without copying them.
+# parameter names, so the engine model is built around the checkpoint's tensors (adopt_state says which of them
+# end up copied).
 
 def _plain(value):
     """Configuration enums of the checkpoint (StrEnum members) and plain strings compare alike."""
@@ -305,8 +313,12 @@ def _engine_dtype(state):
 
 
 def adopt_state(engine_cls, config: LLaDAConfig, state: dict):
-    """An ``engine_cls`` model whose parameters ARE the tensors of ``state`` (no second copy of the weights in
-    device memory; the merged projections the blocks build on first use are the only copies)."""
+    """An ``engine_cls`` model built around the tensors of ``state``.  Embedding, norms, output projections, the
+    MLP down projection and the head ARE those tensors.  The q/k/v and gate/up projections are merged into one
+    weight each (built here, on a GPU, so that a KV cache sized afterwards accounts for them): new tensors of the
+    same total size, so while the caller keeps the checkpoint object these projections (about three quarters of
+    a decoder block, 9.6 GB of LLaDA-8B's 16 GB in bf16) are resident twice.  Floating-point parameters that are
+    not bf16 are converted, which copies them as well."""
     with torch.device("meta"):
         engine = engine_cls(config)
     state = _engine_dtype(state)
@@ -317,6 +329,10 @@ def adopt_state(engine_cls, config: LLaDAConfig, state: dict):
     engine.load_state_dict(state, strict=True, assign=True)
     for p in engine.parameters():
         p.requires_grad_(False)
+    if next(engine.parameters()).is_cuda:
+        with torch.no_grad():
+            for block in engine.model.transformer["blocks"]:
+                block.fuse_projections()
     return engine.eval()
 
 

@@ -64,6 +64,12 @@ class ModelRunner:
         self.last_timing = {}
         self._decode_graph_warm = set()
         self._active_timing = None
+        # the merged projection weights exist before the cache is sized from free device memory
+        if self.device.type == "cuda" and hasattr(self.base_model, "model"):
+            with torch.no_grad():
+                for block in self._llada_blocks():
+                    if hasattr(block, "fuse_projections"):
+                        block.fuse_projections()
         self.allocate_kv_cache()
 
     # ------------------------------------------------------------------ model access
@@ -445,8 +451,12 @@ class ModelRunner:
             cu_q = [0]
             for seq in active_seqs:
                 cu_q.append(cu_q[-1] + len(seq.recompute_positions))
-            mask_rows = input_ids == self.config.mask_id
-            mask_positions = [torch.where(mask_rows[cu_q[b]:cu_q[b + 1]])[0] + cu_q[b] for b in range(len(active_seqs))]
+            # the [MASK] rows of every request among its probe queries, from the host's token lists (the same lists
+            # input_ids was built from): no read-back of a device mask
+            mask_positions = []
+            for b, seq in enumerate(active_seqs):
+                probe_tokens = np.asarray(seq.token_ids, dtype=np.int64)[np.asarray(seq.recompute_positions, dtype=np.int64)]
+                mask_positions.append(np.nonzero(probe_tokens == self.config.mask_id)[0] + cu_q[b])
             self._add_timing_count(timing, "anchor_selection_query_tokens", int(input_ids.numel()))
             self._add_timing_count(timing, "anchor_selection_kv_tokens", sum(len(s) for s in active_seqs))
             self._finish_timing(timing, "anchor_selection_prepare", start)
@@ -454,8 +464,8 @@ class ModelRunner:
             uses_rope = bool(getattr(self.config.hf_config, "rope", True))
             # one kernel pair per layer for the whole batch: softmax over the affix keys of every [MASK] query,
             # column sums over queries and heads added to `importance` (the reference loops over requests here)
-            probe_rows = torch.cat(mask_positions).to(torch.int32)
-            counts = [int(rows.numel()) for rows in mask_positions]
+            counts = [int(rows.size) for rows in mask_positions]
+            probe_rows = self._to_device(np.concatenate(mask_positions) if mask_positions else np.zeros(0), torch.int32)
             probe_cu = self._to_device(np.concatenate([[0], np.cumsum(counts)]), torch.int32)
             shifts = [seq.affix_start if uses_rope else 0 for seq in active_seqs]
             probe_shifts = probe_cos = probe_sin = None
@@ -465,13 +475,13 @@ class ModelRunner:
                     max(self._affix_relocation_max_position, max(shifts) + 1), self.device)
             probe_scratch = torch.empty(
                 max(16, ops.affix_importance_workspace_bytes(
-                    int(probe_rows.numel()), len(active_seqs), blocks[0].attn.num_heads, blocks[0].attn.num_kv_heads,
+                    sum(counts), len(active_seqs), blocks[0].attn.num_heads, blocks[0].attn.num_kv_heads,
                     blocks[0].attn.head_dim, affix_len, probe_shifts is not None)),
                 dtype=torch.uint8, device=self.device)
 
             def make_probe(layer_idx, block):
                 def probe(attention, q):
-                    if probe_rows.numel() == 0:
+                    if sum(counts) == 0:
                         return
                     ops.affix_importance(
                         importance, q.reshape(-1, attention.num_heads, attention.head_dim), attention.k_cache,
@@ -920,12 +930,14 @@ class ModelRunner:
         self._active_timing = timing
         total_start = self._start_timing()
 
-        # positions index the model's rotary table; the kernels clamp an out-of-table row for memory safety only
-        # (it would come back unrotated), so the length is checked here, on the host, where it is known
-        table_rows = getattr(cfg.hf_config, "max_sequence_length", None) or getattr(cfg.hf_config, "max_position_embeddings", None)
+        # Positions index the model's rotary table, and the kernels clamp an out-of-table row for memory safety only
+        # (it would come back unrotated).  The table has no hard limit: like the reference's, which builds it for
+        # position_ids.max() + 1 (nano-vdllm/model/modeling_llada.py:910), it grows to the longest request here,
+        # on the host, where the lengths are known.
         longest = max((len(seq) for seq in prompts), default=0)
-        if table_rows is not None and longest > int(table_rows):
-            raise ValueError(f"a request of {longest} tokens exceeds the model's rotary table of {int(table_rows)} positions")
+        core = getattr(self.base_model, "model", None)
+        if core is not None and hasattr(core, "config"):
+            core.rope_positions = max(int(getattr(core, "rope_positions", 0)), longest)
 
         total_nfe = 0
         results = [None] * len(prompts)
@@ -1006,12 +1018,19 @@ class ModelRunner:
         decoding_positions = None
         decode_graph = None
         stalled = None   # device flag of the last refinement step: it left every [MASK] of its rows in place
+        stalled_steps = 0
+        # At temperature 0 the forward is deterministic: one step without a committed token would repeat for ever.
+        # With sampling the next step draws other tokens, so only a run of such steps is taken as no progress.
+        stall_limit = 1 if temperature == 0 else 8
         while batch:
-            if stalled is not None and bool(stalled):
-                # the committed tokens were all [MASK] again; the same forward would repeat for ever
-                raise RuntimeError(
-                    "Refinement step committed no token: the model predicts the mask token at every position "
-                    "still masked in the active blocks, so block-wise decoding cannot make progress.")
+            if stalled is not None:
+                stalled_steps = stalled_steps + 1 if bool(stalled) else 0
+                if stalled_steps >= stall_limit:
+                    err = RuntimeError(
+                        "Refinement step committed no token: the model predicts the mask token at every position "
+                        "still masked in the active blocks, so block-wise decoding cannot make progress.")
+                    err.partial_results = results   # requests that had finished before the loop gave up
+                    raise err
             stalled = None
             has_mask = (working == mask_id).any(dim=1)
             done = ~has_mask

@@ -455,3 +455,28 @@ def test_merged_projections_keep_the_state_dict_and_follow_parameter_updates(dev
     hook = block.k_proj.register_forward_hook(lambda m, i, o: None)
     torch.testing.assert_close(forward(), changed, rtol=2e-2, atol=2e-2)
     hook.remove()
+
+
+def test_request_longer_than_the_configured_length_is_served(device):
+    """The rotary table grows with the request (the reference builds it for position_ids.max() + 1,
+    nano-vdllm/model/modeling_llada.py:910): a request past ``max_sequence_length`` generates the tokens that the
+    same weights generate under a configuration whose table was long enough from the start."""
+    import copy
+
+    cfg, model = _model(device, seed=3)
+    assert cfg.max_sequence_length == 64
+    wide_cfg = copy.deepcopy(cfg)
+    wide_cfg.max_sequence_length = 256
+    wide = LLaDAModelLM(wide_cfg, init_std=0.08).to(device=device, dtype=torch.bfloat16).eval()
+    wide.load_state_dict(model.state_dict())
+    prompt = [2 + (7 * i) % 50 for i in range(90)]
+
+    def run(m, c):
+        runner = ModelRunner(m, _serve(c, num_kvcache_blocks=32, gen_length=8, anchor_ratio=0.25, threshold=0.9))
+        seq = Sequence(list(prompt), gen_length=8, cache_block_size=8, block_length=4, mask_id=63,
+                       prompt_affix_start=10, prompt_affix_end=50)
+        return runner.generate_with_acache([seq])
+
+    got, nfe = run(model, cfg)
+    want, nfe_want = run(wide, wide_cfg)
+    assert got == want and nfe == nfe_want and 63 not in got[0]

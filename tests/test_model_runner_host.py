@@ -136,6 +136,52 @@ def test_refinement_loop_raises_when_a_step_commits_nothing():
     assert runner.model.calls <= 3   # one refresh forward, one refinement forward, no spin
 
 
+def test_with_sampling_one_step_without_a_commit_is_not_the_end():
+    """temperature > 0: a step in which every draw is [MASK] may be followed by one that commits tokens (the
+    reference keeps looping, model_runner.py:2242-2271); only a run of such steps is given up on, and the error then
+    carries the requests that had finished."""
+    runner = _tiny_runner(num_kvcache_blocks=8, enable_acache=False, threshold=0.9, temperature=0.5)
+    runner.allocate_kv_cache(8)
+    state = {"refinements": 0}
+
+    def rule(tokens):
+        if tokens.dim() == 2:                    # refinement forward: every other one answers [MASK] everywhere
+            state["refinements"] += 1
+            if state["refinements"] % 2 == 1:
+                return torch.full_like(tokens, 63)
+        return torch.full_like(tokens, 7)
+
+    stub = _StubForward(rule)
+    stub_call = stub.__call__
+
+    def peaked(*args, **kwargs):                 # refinement: a head so peaked that the Gumbel draw is its arg-max
+        out = stub_call(*args, **kwargs)
+        if kwargs.get("logits_keep_indices") is None:
+            out.logits = out.logits * 50.0       # (a block refresh stays below the threshold: one forced token per row)
+        return out
+
+    runner.model = peaked
+    torch.manual_seed(0)
+    out, nfe = runner.generate_with_dual_cache(_stub_requests())
+    assert all(len(o) == 8 and 63 not in o for o in out)
+    assert state["refinements"] >= 2
+    # a head that never answers anything else is still given up on, after a bounded number of steps
+    runner2 = _tiny_runner(num_kvcache_blocks=8, enable_acache=False, threshold=0.9, temperature=0.5)
+    runner2.allocate_kv_cache(8)
+    always = _StubForward(lambda tokens: torch.full_like(tokens, 63))
+    always_call = always.__call__
+
+    def peaked_mask(*args, **kwargs):
+        out = always_call(*args, **kwargs)
+        out.logits = out.logits * 50.0
+        return out
+
+    runner2.model = peaked_mask
+    with pytest.raises(RuntimeError, match="committed no token") as info:
+        runner2.generate_with_dual_cache(_stub_requests())
+    assert always.calls <= 1 + 8 + 1 and hasattr(info.value, "partial_results")
+
+
 def test_forced_pick_skips_positions_that_predict_the_mask_token():
     """Column 0 answers [MASK] until the rest of its block is filled, with the same confidence as every other
     position; the forced one-token-per-step pick must take the other positions first and the run must finish."""
@@ -199,16 +245,32 @@ def test_out_of_memory_at_admission_shrinks_retries_and_restores(capsys):
     assert runner.kv_cache.shape[2] == 12
 
 
-def test_requests_longer_than_the_rotary_table_are_refused():
-    """Positions past the model's rotary table would be left unrotated by the kernels (they only clamp for memory
-    safety); the engine refuses such a request on the host before any forward."""
+def test_requests_longer_than_the_configured_length_grow_the_rotary_table():
+    """The reference's rotary table grows with the positions it is asked for (nano-vdllm/model/modeling_llada.py:910);
+    the engine does the same on the host before the first forward instead of leaving out-of-table rows unrotated."""
+    from acache_amd.rope import rope_table
+
     runner = _tiny_runner(num_kvcache_blocks=16, enable_acache=False)
     runner.allocate_kv_cache(16)
-    runner.model = _StubForward(lambda tokens: torch.full_like(tokens, 7))
-    too_long = Sequence(list(range(2, 62)), gen_length=8, cache_block_size=8, block_length=4, mask_id=63)  # 68 > 64
-    with pytest.raises(ValueError, match="rotary table"):
-        runner.generate_with_dual_cache([too_long])
-    assert runner.model.calls == 0
+    core = runner.base_model.model
+    assert core.config.max_sequence_length == 64
+    seen = {}
+
+    def forward(input_ids, position_ids=None, logits_keep_indices=None):
+        seen["rows"] = max(core.config.max_sequence_length, int(getattr(core, "rope_positions", 0)))
+        tokens = input_ids[logits_keep_indices] if logits_keep_indices is not None else input_ids
+        logits = torch.zeros(*tokens.shape, 64)
+        logits[..., 7] = 9.0
+        return SimpleNamespace(logits=logits)
+
+    runner.model = forward
+    long_request = Sequence(list(range(2, 62)), gen_length=8, cache_block_size=8, block_length=4, mask_id=63)  # 68 > 64
+    out, _ = runner.generate_with_dual_cache([long_request])
+    assert out == [[7] * 8] and seen["rows"] == 68
+    # the rotary module hands out as many rows as it is asked for, equal to the closed-form table
+    sin, cos = core.transformer["blocks"][0].rotary_emb.get_rotary_embedding(68, torch.device("cpu"))
+    want_cos, want_sin = rope_table(68, 64, core.config.rope_theta)
+    assert sin.shape[0] == 68 and torch.equal(cos, want_cos) and torch.equal(sin, want_sin)
 
 
 def test_model_runner_takes_over_a_checkpoint_model_object():
