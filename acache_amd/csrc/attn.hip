@@ -17,9 +17,9 @@
 // Two kernels:
 //   varlen_attn_unit_kernel (head_dim 64 and 128, all three relocation modes): K/V rows are copied
 //     global -> LDS directly through the slot map into a two-deep ring, swizzled by permuting the
-//     global side of the copy; V stays row-major and is read with the LDS transpose read.  Queries are
-//     multiplied by scale * log2 e when their fragments are loaded and the score accumulators start
-//     at minus the softmax reference, so a probability is exp2 of its accumulator as it stands.
+//     global side of the copy; V stays row-major and is read with the LDS transpose read.  Scores are
+//     scaled in fp32 inside the softmax (one fused multiply-add per score in front of exp2), as the
+//     reference scales the fp32 product.
 //     Key-side relocation re-rotates the shared rows of a tile in LDS once it has landed.
 //   varlen_attn_kernel (any other head_dim): rows are staged through registers, re-rotated there in
 //     key-side mode, and V is transposed on the way into LDS; scores are scaled in the softmax.
@@ -472,15 +472,6 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
         for (int ks = 0; ks < KS / 2; ++ks)
           rotate_pair<DTYPE, D>(qf[qt][ks], qf[qt][ks + KS / 2], cr, sr, 32 * ks + 8 * lg, -1.0f);
       }
-      // queries are scored as q * scale * log2 e (rounded to the cache type once more), so the scores come out
-      // of the matrix core in the log2 units the softmax works in
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        float f[8];
-        Elem<DTYPE>::unpack(qf[qt][ks], f);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) qf[qt][ks].w[j] = M::pack2(f[2 * j] * p.scale_log2e, f[2 * j + 1] * p.scale_log2e);
-      }
     }
   };
   load_q(MODE == MODE_QUERY_SIDE && t_begin < tiles_a);
@@ -577,14 +568,12 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     }
   };
 
-  // m_run: reference point of the running sums in log2 units; neg_m: minus the value the score accumulators
-  // start at (the reference, or 0 in front of the first tile), replicated as an accumulator operand
+  // m_run: reference point of the running sums in log2 units (score * scale * log2 e)
   float m_run[NQ16];
   f32x4 o_acc[NQ16][DT], l_acc[NQ16];
-  f32x4 neg_m[NQ16];
+  const float c = p.scale_log2e;
 #pragma unroll
   for (int qt = 0; qt < NQ16; ++qt) {
-    neg_m[qt] = f32x4{0, 0, 0, 0};
     m_run[qt] = -INFINITY;
     l_acc[qt] = f32x4{0, 0, 0, 0};
 #pragma unroll
@@ -626,7 +615,7 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
 #pragma unroll
     for (int qt = 0; qt < NQ16; ++qt)
 #pragma unroll
-      for (int nt = 0; nt < NTL; ++nt) s_acc[qt][nt] = neg_m[qt];  // the accumulators start at minus the reference
+      for (int nt = 0; nt < NTL; ++nt) s_acc[qt][nt] = f32x4{0, 0, 0, 0};
     auto scores = [&](const vec16 (&qq)[NQ16][KS]) __attribute__((always_inline)) {
 #pragma unroll
       for (int nt = 0; nt < NTL; ++nt) {
@@ -656,8 +645,7 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
     __builtin_amdgcn_s_setprio(0);
 
     copy_point(1);
-    softmax_reference_prescaled<NQ16, NQ16, NTL, DT, MASKED>(s_acc, m_run, neg_m, l_acc, o_acc,
-                                                             n_valid - kp * (BN / KSPLIT), lg);
+    softmax_reference<NQ16, NQ16, NTL, DT, MASKED>(s_acc, m_run, l_acc, o_acc, c, n_valid - kp * (BN / KSPLIT), lg);
     copy_point(2);
 
     // O^T += V^T P^T, one 32-key slab at a time, so that the exponentials of the second slab
@@ -678,12 +666,12 @@ __device__ __forceinline__ void attn_dma_part(const AttnParams &p, char *lds_k0,
           o_acc[qt][dt] = M::run(vf, pf[qt][s], o_acc[qt][dt]);
       }
     };
-    softmax_probs_slab_prescaled<M, 0, NQ16>(s_acc, l_acc, pf, ones);
+    softmax_probs_slab<M, 0, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
     copy_point(3);
     __builtin_amdgcn_s_setprio(1);
     pv_slab(0);  // with a key split this is the wave's own slab: its offset is part of v_frag
     if constexpr (NSL == 2) {
-      softmax_probs_slab_prescaled<M, 1, NQ16>(s_acc, l_acc, pf, ones);
+      softmax_probs_slab<M, 1, NQ16>(s_acc, m_run, l_acc, pf, ones, c);
       pv_slab(1);
     }
     // Issue order: V fragments two d-tiles ahead of their use.

@@ -241,7 +241,9 @@ __device__ __forceinline__ void softmax_reference(f32x4 (&s_acc)[NQ16][NT], floa
     // its wave (workgroups may give a wave one or two such tiles).  Every lane tests the maximum of its own
     // keys: the ballot is true exactly when some query's maximum over the whole tile exceeds the bound, so the
     // cross-lane maximum (two LDS round trips) is only taken when the reference really moves.
-    if (__builtin_amdgcn_ballot_w64(mx * c > m_run[qt] + 8.0f) != 0) {
+    // (a first tile without any present key still moves the reference off -inf, to 0, so that the
+    // probabilities below come out as exp2(-inf) = 0 rather than exp2(-inf + inf))
+    if (__builtin_amdgcn_ballot_w64(mx * c > m_run[qt] + 8.0f || m_run[qt] == -INFINITY) != 0) {
       mx = fmaxf(mx, __shfl_xor(mx, 16));
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float mxc = mx * c;
@@ -272,67 +274,6 @@ __device__ __forceinline__ void softmax_probs_slab(const f32x4 (&s_acc)[NQ16][NT
 #pragma unroll
     // one fused multiply-add per score (contraction is switched off for this library, so it is asked for by name)
     for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[qt][2 * S + (j >> 2)][j & 3], c, -mc));
-    pf[qt][S].w[0] = M::pack2(e[0], e[1]);
-    pf[qt][S].w[1] = M::pack2(e[2], e[3]);
-    pf[qt][S].w[2] = M::pack2(e[4], e[5]);
-    pf[qt][S].w[3] = M::pack2(e[6], e[7]);
-    l_acc[qt] = M::run(ones, pf[qt][S], l_acc[qt]);
-  }
-}
-
-// The same two steps for a kernel whose queries were multiplied by scale * log2 e when their fragments were
-// loaded and whose score accumulators start at minus the reference (neg_m, the reference replicated over the
-// four elements of an accumulator, 0 while m_run is still -inf): s_acc arrives as score * scale * log2 e - m_run,
-// the probability is exp2 of it as it stands, and the multiply-add per score is gone.  When the reference
-// moves, the tile's accumulators are re-based as well.
-template <int NQA, int NQ16, int NT, int DT, bool MASKED>
-__device__ __forceinline__ void softmax_reference_prescaled(f32x4 (&s_acc)[NQ16][NT], float (&m_run)[NQ16],
-                                                            f32x4 (&neg_m)[NQ16], f32x4 (&l_acc)[NQ16],
-                                                            f32x4 (&o_acc)[NQ16][DT], int n_valid, int lg) {
-  static_assert(NQA <= NQ16, "live query tiles");
-#pragma unroll
-  for (int qt = 0; qt < NQA; ++qt) {
-    if (MASKED && n_valid < 16 * NT) {  // wave-uniform: full tiles skip the masking code
-      const int limit = n_valid - 4 * lg;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (16 * nt + i >= limit) s_acc[qt][nt][i] = -INFINITY;
-    }
-    float mx = -INFINITY;
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s_acc[qt][nt][i]);
-    // the first tile always sets the reference (all lanes of a wave leave -inf together)
-    if (__builtin_amdgcn_ballot_w64(mx > 8.0f || m_run[qt] == -INFINITY) != 0) {
-      mx = fmaxf(mx, __shfl_xor(mx, 16));
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_old = -neg_m[qt][0];              // the value the accumulators are relative to
-      const float m_new = fmaxf(m_run[qt], mx + m_old);
-      const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m_run[qt] - m_use);
-      const float shift = m_use - m_old;
-      l_acc[qt] *= alpha;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) o_acc[qt][dt] *= alpha;
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) s_acc[qt][nt] -= shift;
-      m_run[qt] = m_use;
-      neg_m[qt] = f32x4{-m_use, -m_use, -m_use, -m_use};
-    }
-  }
-}
-
-template <class M, int S, int NQA, int NQ16, int NT, int NS>
-__device__ __forceinline__ void softmax_probs_slab_prescaled(const f32x4 (&s_acc)[NQ16][NT], f32x4 (&l_acc)[NQ16],
-                                                             vec16 (&pf)[NQ16][NS], const vec16 &ones) {
-#pragma unroll
-  for (int qt = 0; qt < NQA; ++qt) {
-    float e[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s_acc[qt][2 * S + (j >> 2)][j & 3]);
     pf[qt][S].w[0] = M::pack2(e[0], e[1]);
     pf[qt][S].w[1] = M::pack2(e[2], e[3]);
     pf[qt][S].w[2] = M::pack2(e[4], e[5]);

@@ -328,10 +328,9 @@ int acache_build_slot_layout(
  *     K_b[n] = k_cache[slot_map[cu_k[b] + n], kv head],  V_b[n] likewise
  *     out[cu_q[b] + m, h] = softmax_n(q[cu_q[b] + m, h] . K_b[n] * scale) . V_b
  *   fp32 accumulation, probabilities rounded to `dtype` before the PV product,
- *   output rounded to `dtype`.  At head_dim 64 / 128 the scale is applied to the
- *   query (q * scale * log2 e rounded to `dtype`, exp2 of the fp32 product) where
- *   the reference scales the fp32 product (lines 439, 460, 499): one more rounding of q, within
- *   the 2e-2 absolute bound on outputs the parity tests hold this call to.
+ *   output rounded to `dtype`.  The scale is applied to the fp32 product, as the reference does
+ *   (lines 439, 460, 499): scores of any magnitude keep the 2e-2 absolute bound on outputs that the
+ *   parity tests hold this call to.
  *
  * Relocation modes (selected exactly as the reference wrapper does,
  * nano-vdllm/model/acache_attention.py:670-671):

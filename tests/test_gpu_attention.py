@@ -430,3 +430,48 @@ def test_relocation_argument_errors(device):
     cos = torch.ones(8, 64, device=device)
     with pytest.raises(ValueError, match="provided together"):
         ops.acache_attention(q, kc, kc, cu, cu, slots, rope_cos=cos)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_near_ties_among_large_scores(device, D):
+    """The head-dim 64 / 128 kernels score q * scale * log2 e, rounded to the cache type once more, where the
+    reference scales the fp32 product (acache_attention.py:439, 460, 499).  Here every query is aligned with TWO
+    keys, so two scores of magnitude 30 compete and their difference (of order one) decides the output: the case in
+    which an error relative to the score's size shows most.  Same bound as everywhere else."""
+    g = torch.Generator().manual_seed(11)
+    H, S, n_q, n_kv = 4, 512, 90, 300
+    kc = torch.randn(S, H, D, generator=g)
+    kc = (kc / kc.norm(dim=-1, keepdim=True)).to(torch.bfloat16)              # unit keys
+    vc = torch.randn(S, H, D, generator=g).to(torch.bfloat16)
+    slots = torch.randperm(S, generator=g)[:n_kv].to(torch.int32)
+    first = slots[torch.randint(0, n_kv, (n_q,), generator=g)].long()
+    second = slots[torch.randint(0, n_kv, (n_q,), generator=g)].long()
+    # 30 / scale along both keys plus noise: both score ~30 (+- 1), every other key ~N(0, 1)
+    q = ((kc[first].float() + kc[second].float()) * (30.0 * D ** 0.5) + torch.randn(n_q, H, D, generator=g)).to(torch.bfloat16)
+    cu_q = torch.tensor([0, n_q], dtype=torch.int32)
+    cu_k = torch.tensor([0, n_kv], dtype=torch.int32)
+    want = O.acache_attention(q, kc.view(S // 16, 16, H, D), vc.view(S // 16, 16, H, D), cu_q, cu_k, slots)
+    scores = torch.einsum("qhd,khd->hqk", q.float(), kc[slots.long()].float()) * D ** -0.5
+    top2 = scores.topk(2, dim=-1).values
+    assert top2[..., 1].median().item() > 25.0 and (top2[..., 0] - top2[..., 1]).median().item() < 3.0
+    got = ops.acache_attention(q.to(device), kc.view(S // 16, 16, H, D).to(device), vc.view(S // 16, 16, H, D).to(device),
+                               cu_q.to(device), cu_k.to(device), slots.to(device))
+    _close(got, want)
+
+
+def test_f16_queries_of_small_magnitude(device):
+    """f16: queries of magnitude 1e-3 times the scale land near the bottom of the normal range when they are
+    pre-scaled; keys of magnitude 1e2 keep the scores of order one, so lost query bits would show.  Same bound."""
+    g = torch.Generator().manual_seed(12)
+    H, Hkv, D, S, n_q, n_kv = 4, 2, 128, 512, 70, 260
+    q = (torch.randn(n_q, H, D, generator=g) * 1e-3).to(torch.float16)
+    kc = (torch.randn(S, Hkv, D, generator=g) * 1e2).to(torch.float16)
+    vc = torch.randn(S, Hkv, D, generator=g).to(torch.float16)
+    slots = torch.randperm(S, generator=g)[:n_kv].to(torch.int32)
+    cu_q = torch.tensor([0, n_q], dtype=torch.int32)
+    cu_k = torch.tensor([0, n_kv], dtype=torch.int32)
+    want = O.acache_attention(q, kc.view(S // 16, 16, Hkv, D), vc.view(S // 16, 16, Hkv, D), cu_q, cu_k, slots)
+    got = ops.acache_attention(q.to(device), kc.view(S // 16, 16, Hkv, D).to(device),
+                               vc.view(S // 16, 16, Hkv, D).to(device), cu_q.to(device), cu_k.to(device), slots.to(device))
+    assert (q.float().abs().max() * D ** -0.5 * 1.4427).item() < 1e-3      # pre-scaled values: a few 1e-4
+    _close(got, want)
