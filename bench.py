@@ -411,6 +411,25 @@ def attention_shape_sweep(torch, device, ops, steps):
         kv_bytes = 2 * S * Hkv * D * 2
         rows.append({"B": B, "q": q, "kv": kv, "H": H, "H_kv": Hkv, "us": round(ms * 1e3, 1),
                      "TFLOPs": round(4 * H * D * B * q * kv / ms / 1e9, 0), "kv_GBps": round(kv_bytes / ms / 1e6, 0)})
+    # Decode shapes as the engine issues them: the non-anchor affix rows of every request are the SAME slots (L2 hits
+    # after the first request), only the anchors, the request text and the generation window are private rows.
+    shared_rows = []
+    for B, q, kv, shared, H, Hkv in ((16, 32, 1400, 1000, 32, 32), (16, 32, 1400, 800, 32, 32), (16, 32, 1400, 1000, 28, 4)):
+        S = shared + B * (kv - shared)
+        Q = (torch.randn(B * q, H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        K = (torch.randn(S, 1, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        V = (torch.randn(S, 1, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        cu_q = torch.arange(0, (B + 1) * q, q, dtype=torch.int32, device=device)
+        cu_k = torch.arange(0, (B + 1) * kv, kv, dtype=torch.int32, device=device)
+        common = torch.arange(shared, dtype=torch.int32)
+        slots = torch.cat([torch.cat([common, torch.arange(shared + b * (kv - shared), shared + (b + 1) * (kv - shared),
+                                                           dtype=torch.int32)]) for b in range(B)]).to(device)
+        for _ in range(3):
+            ops.acache_attention(Q, K, V, cu_q, cu_k, slots)
+        ms = _event_times_ms(lambda: ops.acache_attention(Q, K, V, cu_q, cu_k, slots), steps, torch)[0]
+        shared_rows.append({"B": B, "q": q, "kv": kv, "shared_kv": shared, "H": H, "H_kv": Hkv, "us": round(ms * 1e3, 1),
+                            "distinct_kv_GBps": round(2 * S * Hkv * D * 2 / ms / 1e6, 0),
+                            "streamed_kv_GBps": round(2 * B * kv * Hkv * D * 2 / ms / 1e6, 0)})
     # The three relocation modes on one relocated anchor-recompute shape: batch 16, 232 queries and 1 400 keys per
     # request, a shared affix of 1 000 slots placed 50 + 10 b positions into request b (back-to-back launches).
     from acache_amd.rope import rope_table
@@ -440,7 +459,8 @@ def attention_shape_sweep(torch, device, ops, steps):
             call()
         ms = _event_times_ms(call, steps, torch)[0]
         modes.append({"mode": name, "us": round(ms * 1e3, 1), "TFLOPs": round(flops / ms / 1e9, 0)})
-    print(json.dumps({"attention_shape_sweep": rows, "relocation_modes": modes}))
+    print(json.dumps({"attention_shape_sweep": rows, "decode_shapes_with_shared_affix_rows": shared_rows,
+                      "relocation_modes": modes}))
 
 
 def kernel_sweep(torch, device, ops, steps):
