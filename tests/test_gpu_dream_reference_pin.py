@@ -240,11 +240,31 @@ def test_engine_logits_match_the_restated_dream_forward(device, seed):
     want, _ = TorchDream(sd).forward(torch.tensor(tokens), torch.arange(len(tokens)))
     got = _engine_dense_logits(model, tokens).cpu()
     assert got.shape == want.shape
-    # the reference's own bound for engine logits (tests/test_model_runner_acache.py:687: rtol = atol = 5e-2); a
-    # swapped projection pair or a wrong rotary convention is off by the size of the logits themselves
-    torch.testing.assert_close(got, want, rtol=5e-2, atol=5e-2)
-    assert (got - want).abs().mean().item() <= 2e-2
+    # bf16 engine against an fp32 model: the rounding of two layers of bf16 activations shows in full (the
+    # reference's own engine tests compare bf16 with bf16 at rtol = atol = 5e-2, tests/test_model_runner_acache.py:687).
+    # Measured: mean 1.3e-2, largest 7.5e-2 on logits of magnitude up to 5.
+    diff = (got - want).abs()
+    assert diff.mean().item() <= 2e-2 and diff.max().item() <= 1.5e-1, (diff.mean().item(), diff.max().item())
     assert want.abs().max().item() > 1.0      # the comparison is not vacuous: logits of order one
+    # ... and the bound has teeth: the same forward with one pair of projections exchanged (what a slip in the
+    # checkpoint name mapping would do) or with the rotary halves the other way round is far outside it
+    for a, b in (("mlp.gate_proj", "mlp.up_proj"), ("self_attn.k_proj", "self_attn.v_proj")):
+        swapped = dict(sd)
+        for key in sd:
+            if a in key:
+                swapped[key], swapped[key.replace(a, b)] = sd[key.replace(a, b)], sd[key]
+        wrong, _ = TorchDream(swapped).forward(torch.tensor(tokens), torch.arange(len(tokens)))
+        assert (got - wrong).abs().mean().item() > 10 * 2e-2, (a, b)
+    shifted, _ = TorchDream(sd).forward(torch.tensor(tokens), torch.arange(len(tokens)) + 3)
+    assert (shifted - want).abs().max().item() < 1e-3     # rotary positions are relative: a uniform offset changes nothing
+    flipped = TorchDream(sd)
+    flipped.inv_freq = -flipped.inv_freq                                  # the rotation the other way round ...
+    wrong, _ = flipped.forward(torch.tensor(tokens), torch.arange(len(tokens)))
+    assert (got - wrong).abs().mean().item() > 10 * 2e-2  # ... swaps left and right context: a different model
+    nope = TorchDream(sd)
+    nope._rope = lambda x, positions: x                                   # and so is no rotary at all
+    wrong, _ = nope.forward(torch.tensor(tokens), torch.arange(len(tokens)))
+    assert (got - wrong).abs().mean().item() > 10 * 2e-2
 
 
 @pytest.mark.parametrize("placement", ["prefix", "infix", "suffix"])
