@@ -73,10 +73,11 @@ class TorchDream:
         x1, x2 = x[..., : HD // 2], x[..., HD // 2:]
         return x * cos + torch.cat((-x2, x1), dim=-1) * sin
 
-    def forward(self, tokens, positions, cache=None, replace_rows=None):
+    def forward(self, tokens, positions, cache=None, replace_rows=None, probe=None):
         """tokens, positions: [T].  cache: per layer (k, v) [L, HKV * HD] before RoPE, rows at absolute positions
         0..L-1; the T inputs overwrite rows ``replace_rows`` (one to one).  Without a cache the inputs are the
-        whole sequence.  Returns (logits [T, V], cache)."""
+        whole sequence.  ``probe(layer, q)`` sees every layer's queries before RoPE, ``[T, H, HD]``.
+        Returns (logits [T, V], cache)."""
         sd = self.sd
         x = sd["model.embed_tokens.weight"][tokens]
         new_cache = []
@@ -84,6 +85,8 @@ class TorchDream:
             p = f"model.layers.{i}."
             y = self._rms(x, sd[p + "input_layernorm.weight"])
             q = F.linear(y, sd[p + "self_attn.q_proj.weight"], sd[p + "self_attn.q_proj.bias"])
+            if probe is not None:
+                probe(i, q.view(-1, H, HD))
             k = F.linear(y, sd[p + "self_attn.k_proj.weight"], sd[p + "self_attn.k_proj.bias"])
             v = F.linear(y, sd[p + "self_attn.v_proj.weight"], sd[p + "self_attn.v_proj.bias"])
             if cache is None:
@@ -297,3 +300,132 @@ def test_all_anchor_generation_equals_the_restated_loop(device, placement, mode)
     assert nfe == nfe_want                      # no importance pass is counted when every affix token is an anchor
     if mode == "quota":
         assert nfe == 8                         # per block of four: one refresh (seeds one token) + three quota steps
+
+
+# --------------------------------------------------------------------------------------------------------------
+# Anchor ratio below 1: the path that actually reuses the affix.  Restated from dream/generate_ACache.py:
+#   the affix cache is the affix ALONE at positions 0..A-1, keys before RoPE (acache_eval_shared.py:599-609);
+#   importance (183-344): one forward over the non-affix tokens against a cache that holds the frozen affix rows;
+#     per layer, softmax over the AFFIX keys only of every query (rotated at their absolute positions), summed
+#     over heads and over the [MASK] queries;
+#   anchors (347-375): top-k by importance, ascending, plus affix_start;  k = min(ceil(ratio * A), A) (40-44, 552-553);
+#   recomputed positions = anchors + every non-affix position; logits are shifted left in THAT compact order
+#     (576-628); non-anchor affix rows keep the cached K/V for the whole run.
+
+def reference_affix_cache(model, affix_tokens):
+    _, cache = model.forward(torch.tensor(affix_tokens), torch.arange(len(affix_tokens)))
+    return cache
+
+
+def reference_importance(model, x, affix_cache, a0, A):
+    L = x.numel()
+    probe_pos = torch.cat([torch.arange(0, a0), torch.arange(a0 + A, L)])
+    mask_q = (x[probe_pos] == MASK).float()
+    cache = []
+    for k, v in affix_cache:
+        ck, cv = torch.zeros(L, HKV * HD), torch.zeros(L, HKV * HD)
+        ck[a0:a0 + A], cv[a0:a0 + A] = k, v
+        cache.append((ck, cv))
+    importance = torch.zeros(A)
+
+    def probe(layer, q):                                                  # 246-285
+        q_rot = model._rope(q.transpose(0, 1), probe_pos)                 # [H, T, HD] at the queries' own positions
+        k_rot = model._rope(affix_cache[layer][0].view(A, HKV, HD).transpose(0, 1), torch.arange(a0, a0 + A))
+        k_rot = k_rot.repeat_interleave(H // HKV, dim=0)
+        weights = torch.softmax(q_rot @ k_rot.transpose(1, 2) * HD ** -0.5, dim=-1)       # over affix keys only
+        importance.add_((weights * mask_q[None, :, None]).sum(dim=1).sum(dim=0))
+
+    model.forward(x[probe_pos], probe_pos, cache, probe_pos, probe=probe)
+    return importance
+
+
+def reference_generate_partial(model, prompt, a0, A, ratio, steps, gen_length, block_length, threshold=None):
+    """Returns (x, nfe, anchors, smallest decision margin).  Tail generation (generation_start = len(prompt))."""
+    num_blocks = gen_length // block_length
+    spb = steps // num_blocks
+    gen0 = len(prompt)
+    x = torch.tensor(list(prompt) + [MASK] * gen_length)
+    L = x.numel()
+    affix_cache = reference_affix_cache(model, list(prompt[a0:a0 + A]))
+    k = min(math.ceil(ratio * A), A)
+    importance = reference_importance(model, x, affix_cache, a0, A)
+    ranked = importance.sort(descending=True)
+    anchors = (ranked.indices[:k].sort().values + a0)                     # 367-373 + 571
+    margins = [float(ranked.values[k - 1] - ranked.values[k]) / (0.03 * float(ranked.values[k - 1]))]
+    nfe = 1
+    keep = torch.ones(L, dtype=torch.bool)
+    keep[a0:a0 + A] = False
+    keep[anchors] = True
+    rec = keep.nonzero()[:, 0]                                            # recompute positions, ascending
+    compact_of = {int(pos): i for i, pos in enumerate(rec)}
+    cache = []
+    for ck, cv in affix_cache:                                            # 612-626
+        fk, fv = torch.zeros(L, HKV * HD), torch.zeros(L, HKV * HD)
+        fk[a0:a0 + A], fv[a0:a0 + A] = ck, cv
+        cache.append((fk, fv))
+    logits, cache = model.forward(x[rec], rec, cache, rec)                # 630-640
+    logits, nfe = _align(logits), nfe + 1
+    for nb in range(num_blocks):
+        s = gen0 + nb * block_length
+        e = s + block_length
+        if nb > 0:                                                        # 655-675
+            logits, cache = model.forward(x[rec], rec, cache, rec)
+            logits, nfe = _align(logits), nfe + 1
+        c0 = compact_of[s]
+        blk = logits[c0:c0 + block_length]
+        top2 = blk[0].topk(2).values
+        margins.append(float(top2[0] - top2[1]) / LOGIT_TOL)
+        x[s] = blk[0].argmax()
+        quota = _num_transfer_tokens(x[s:e] == MASK, spb - 1) if threshold is None and spb > 1 else None
+        for i in range(1, spb):
+            if (x[s:e] == MASK).sum() == 0:
+                break
+            out, cache = model.forward(x[s:e], torch.arange(s, e), cache, torch.arange(s, e))
+            nfe += 1
+            x0, transfer, m = _transfer_index(_align(out), x[s:e] == MASK, x[s:e], None if quota is None else quota[i - 1], threshold)
+            margins += m
+            x[s:e] = torch.where(transfer, x0, x[s:e])
+    return x, nfe, anchors.tolist(), min(margins)
+
+
+@pytest.mark.parametrize("placement", ["prefix", "infix"])
+def test_partial_ratio_generation_equals_the_restated_loop(device, placement):
+    """Anchor ratio 0.25: importance pass, top-k anchors, frozen non-anchor affix rows, recompute of anchors and
+    non-affix tokens at every block boundary.  Tokens and forward count must equal the restated reference loop, with
+    the engine's own affix precompute and with the affix cache in Dream's layout handed in."""
+    A = 24
+    affix = [10 + (5 * i) % 40 for i in range(A)]
+    if placement == "prefix":
+        prompt, a0 = affix + [3, 4, 5, 6, 7], 0
+    else:
+        prompt, a0 = [3, 4, 5] + affix + [6, 7, 8], 3
+    for seed in range(400):
+        sd = _checkpoint_state(seed)
+        ref = TorchDream(sd)
+        want, nfe_want, anchors, margin = reference_generate_partial(ref, prompt, a0, A, 0.25, steps=8, gen_length=8,
+                                                                    block_length=4)
+        if margin > 1.0 and len(set(want[-8:].tolist())) >= 4:            # decisive and not one token eight times
+            break
+    else:
+        pytest.fail("no seed with comfortable decision margins")
+    assert len(anchors) == 6 and (want != MASK).all()
+    # the frozen affix rows matter: recomputing the whole affix (every token an anchor) decodes other tokens
+    everything, _, _ = reference_generate(ref, prompt, steps=8, gen_length=8, block_length=4, threshold=None,
+                                          generation_start=None)
+    assert everything.tolist() != want.tolist()
+    model = _engine_model(sd, device)
+    kw = dict(steps=8, gen_length=8, block_length=4, mask_id=MASK, anchor_ratio=0.25, affix_start=a0, affix_end=a0 + A)
+    got, nfe = GD.generate_with_anchor_attention(model, torch.tensor([prompt], device=device), **kw)
+    assert got[0].cpu().tolist() == want.tolist() and nfe == nfe_want
+    # the same call with the reference-layout affix cache: [1, A, H_kv * D] per layer, keys before RoPE
+    cache = tuple((k.to(device=device, dtype=torch.bfloat16)[None], v.to(device=device, dtype=torch.bfloat16)[None])
+                  for k, v in reference_affix_cache(ref, affix))
+    got2, nfe2 = GD.generate_with_anchor_attention(model, torch.tensor([prompt], device=device),
+                                                   precomputed_affix_cache=cache, **kw)
+    assert got2[0].cpu().tolist() == want.tolist() and nfe2 == nfe_want
+    # and the importance values themselves (fp32 there, bf16 with the rotation on the queries here)
+    x = torch.tensor([list(prompt) + [MASK] * 8], device=device)
+    imp = GD.compute_attention_importance_cross_affix(model, x, cache, mask_id=MASK, affix_start=a0).cpu()[0]
+    want_imp = reference_importance(ref, x[0].cpu(), reference_affix_cache(ref, affix), a0, A)
+    torch.testing.assert_close(imp, want_imp, rtol=6e-2, atol=6e-2)
+    assert abs(imp.sum().item() - want_imp.sum().item()) <= 1e-2 * want_imp.sum().item()
