@@ -64,6 +64,15 @@ SIGNATURES = {
         c_int32, c_int32, c_int32, c_int32, c_int64,
         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
         c_void_p]),
+    "acache_varlen_attn_planned": (c_int32, [
+        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+        c_float,
+        c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int32,
+        c_int32, c_int64, c_int64,
+        c_int32, c_int32, c_int32, c_int32, c_int64,
+        c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+        c_void_p, c_int64, c_void_p]),
+    "acache_varlen_attn_plan": (c_int64, [c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_void_p, c_int64]),
 }
 
 

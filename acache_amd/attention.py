@@ -65,6 +65,7 @@ class Attention(nn.Module):
                 context.shared_kv_lens, context.affix_shifts,
                 self.relocation_rope_cos if self.relocation_rope_cos.numel() else None,
                 self.relocation_rope_sin if self.relocation_rope_sin.numel() else None,
+                plan=context.attention_plan,
             )
             return o.view(bs, seqlen, self.num_heads, self.head_dim) if q.dim() == 4 else o
         if context.is_caching:
@@ -72,11 +73,13 @@ class Attention(nn.Module):
                 # fresh (unpaged) q, k, v: identity slot map over the rows just computed
                 total = k.shape[0]
                 slots = torch.arange(total, dtype=torch.int32, device=k.device)
-                return ops.acache_attention(q, k, v, context.cu_seqlens_q, context.cu_seqlens_k, slots, scale)
+                return ops.acache_attention(q, k, v, context.cu_seqlens_q, context.cu_seqlens_k, slots, scale,
+                                            plan=context.attention_plan)
             total_k = getattr(context, "total_k", None)
             return ops.baseline_ragged_attention(
                 q, k_cache, v_cache, context.cu_seqlens_q, context.cu_seqlens_k, context.block_tables,
-                scale, total_k=total_k if total_k is not None else int(context.cu_seqlens_k[-1].item()))
+                scale, total_k=total_k if total_k is not None else int(context.cu_seqlens_k[-1].item()),
+                plan=context.attention_plan)
         q4 = q if q.dim() == 4 else q.view(-1, 1, self.num_heads, self.head_dim)
         total_k = getattr(context, "total_k", None)
         return ops.baseline_decode_attention(q4, k_cache, v_cache, context.seqlens, context.block_tables, scale,

@@ -904,11 +904,27 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
   char *const lds_k0 = lds, *const lds_v0 = lds + TILE_BYTES;
   char *const lds_k1 = lds + 2 * TILE_BYTES, *const lds_v1 = lds + 3 * TILE_BYTES;
   int tile, kvh, hg;
-  if (!block_to_tile_head(p, tile, kvh, hg)) return;
   const int group = p.H / p.H_kv;
-  const int head = kvh * group + hg;
   int b = 0, q_begin = 0, q_len = 0, kv_begin = 0, kv_len = 0;
-  {
+  if (p.plan) {
+    // The caller's dispatch plan names this block's unit.  Every field is checked against the call's own
+    // sizes, so a plan made for other lengths can leave rows unwritten but cannot send an access astray.
+    const int2 e = reinterpret_cast<const int2 *>(p.plan)[blockIdx.x];
+    b = __builtin_amdgcn_readfirstlane(e.x);
+    const unsigned th = (unsigned)__builtin_amdgcn_readfirstlane(e.y);
+    if ((unsigned)b >= (unsigned)p.B) return;
+    tile = (int)(th & 0xfffffu);
+    const int planned_head = (int)(th >> 20);
+    if (planned_head >= p.H) return;
+    kvh = planned_head / group;
+    hg = planned_head - kvh * group;
+    q_begin = p.cu_q[b];
+    q_len = p.cu_q[b + 1] - q_begin;
+    kv_begin = p.cu_k[b];
+    kv_len = p.cu_k[b + 1] - kv_begin;
+    if (tile * BM >= q_len) return;
+  } else {
+    if (!block_to_tile_head(p, tile, kvh, hg)) return;
     int tile_in_request = 0;
     if (p.B <= 64) {
       if (!locate_query_tile_lpt(p.cu_q, p.cu_k, p.B, BM, tile, b, q_begin, q_len, tile_in_request, kv_begin, kv_len)) return;
@@ -919,6 +935,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
     }
     tile = tile_in_request;
   }
+  const int head = kvh * group + hg;
   const int q_tile0 = tile * BM;
   const int kt = sk_key_tiles<MODE>(p, b, kv_len);
   // tiles with at most 64 (32) live rows: two waves per 32 (16) rows, each on half of every tile's keys
@@ -934,11 +951,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void varlen_attn_unit_ker
 }
 
 template <int DTYPE, int D, int NQ16>
-static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, hipStream_t stream) {
+static int launch_attn(const AttnParams &p0, int mode, int64_t total_q, int64_t plan_blocks, hipStream_t stream) {
   AttnParams p = p0;
   // One 4-wave workgroup per (request, 128-row query tile, head), two workgroups per CU.
   p.num_tiles = (int32_t)((total_q + 127) / 128) + p.B;
-  const int64_t blocks = attn_grid_blocks(p);
+  const int64_t blocks = p.plan ? plan_blocks : attn_grid_blocks(p);
   if (blocks > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "varlen_attn: grid too large");
   // 32-bit copy offsets when the whole cache lies within 4 GiB of a head's base and the factors fit 24 bits
   const bool small = p.num_slots < (1 << 24) && p.kv_slot_bytes > 0 && p.kv_slot_bytes < (1 << 24) &&
@@ -989,14 +1006,16 @@ static int launch_attn_any_head_dim(const AttnParams &p0, int mode, int64_t tota
 
 using namespace acache;
 
-extern "C" int acache_varlen_attn(
+extern "C" int acache_varlen_attn_planned(
     void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *cu_q,
     const int32_t *cu_k, const int32_t *slot_map, float scale, int32_t shared_prefix_len,
     const int32_t *shared_kv_lens, const int32_t *affix_shifts, const float *rope_cos,
     const float *rope_sin, int32_t rope_rows, int32_t B, int64_t total_q, int64_t total_k, int32_t H,
     int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t q_token_stride,
     int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t kv_slot_stride,
-    int64_t kv_head_stride, void *stream) {
+    int64_t kv_head_stride, const int32_t *plan, int64_t plan_blocks, void *stream) {
+  if (plan && (plan_blocks <= 0 || ((uintptr_t)plan & 7)))
+    return fail(ACACHE_E_SHAPE, "varlen_attn: a plan needs a positive block count and 8-byte alignment");
   if (dtype != ACACHE_BF16 && dtype != ACACHE_F16)
     return fail(ACACHE_E_DTYPE, "varlen_attn: dtype %d not supported (bf16 or f16)", dtype);
   if (D < 16 || D > 256 || D % 16 != 0)
@@ -1024,6 +1043,7 @@ extern "C" int acache_varlen_attn(
   p.cu_q = cu_q; p.cu_k = cu_k; p.slot_map = slot_map;
   p.shared_kv_lens = shared_kv_lens; p.affix_shifts = affix_shifts;
   p.cos_tab = rope_cos; p.sin_tab = rope_sin;
+  p.plan = (D == 128 || D == 64) ? plan : nullptr;  // the padded-width kernel keeps its own order
   p.scale_log2e = scale * 1.4426950408889634f;
   p.shared_prefix_len = relocate ? shared_prefix_len : 0;
   p.rope_rows = rope_rows; p.B = B; p.H = H; p.H_kv = H_kv; p.num_tiles = 0; p.head_dim = D;
@@ -1034,7 +1054,7 @@ extern "C" int acache_varlen_attn(
   const int mode = query_side ? MODE_QUERY_SIDE : (relocate ? MODE_KEY_SIDE : MODE_PLAIN);
   hipStream_t st = (hipStream_t)stream;
 #define ACACHE_ATTN(DT, DD) \
-  if (dtype == DT && D == DD) return launch_attn<DT, DD, 2>(p, mode, total_q, st);
+  if (dtype == DT && D == DD) return launch_attn<DT, DD, 2>(p, mode, total_q, plan_blocks, st);
   ACACHE_ATTN(ACACHE_BF16, 128)
   ACACHE_ATTN(ACACHE_BF16, 64)
   ACACHE_ATTN(ACACHE_F16, 128)
@@ -1042,4 +1062,18 @@ extern "C" int acache_varlen_attn(
 #undef ACACHE_ATTN
   if (dtype == ACACHE_BF16) return launch_attn_any_head_dim<ACACHE_BF16>(p, mode, total_q, st);
   return launch_attn_any_head_dim<ACACHE_F16>(p, mode, total_q, st);
+}
+
+extern "C" int acache_varlen_attn(
+    void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *cu_q,
+    const int32_t *cu_k, const int32_t *slot_map, float scale, int32_t shared_prefix_len,
+    const int32_t *shared_kv_lens, const int32_t *affix_shifts, const float *rope_cos,
+    const float *rope_sin, int32_t rope_rows, int32_t B, int64_t total_q, int64_t total_k, int32_t H,
+    int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots, int64_t q_token_stride,
+    int64_t q_head_stride, int64_t out_token_stride, int64_t out_head_stride, int64_t kv_slot_stride,
+    int64_t kv_head_stride, void *stream) {
+  return acache_varlen_attn_planned(out, q, k_cache, v_cache, cu_q, cu_k, slot_map, scale, shared_prefix_len,
+                                    shared_kv_lens, affix_shifts, rope_cos, rope_sin, rope_rows, B, total_q, total_k,
+                                    H, H_kv, D, dtype, num_slots, q_token_stride, q_head_stride, out_token_stride,
+                                    out_head_stride, kv_slot_stride, kv_head_stride, nullptr, 0, stream);
 }

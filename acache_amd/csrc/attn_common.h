@@ -26,6 +26,7 @@ struct AttnParams {
   const int32_t *affix_shifts;
   const float *cos_tab;
   const float *sin_tab;
+  const int32_t *plan;  // optional dispatch plan: (request, tile | head << 20) per block, or NULL
   float scale_log2e;
   int32_t shared_prefix_len;
   int32_t rope_rows;

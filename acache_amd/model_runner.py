@@ -64,6 +64,10 @@ class ModelRunner:
         self.last_timing = {}
         self._decode_graph_warm = set()
         self._active_timing = None
+        self._attention_plans = {}
+        # two four-wave workgroups of the attention kernel fit a CU; an XCD holds an eighth of the CUs
+        cus = torch.cuda.get_device_properties(self.device).multi_processor_count if self.device.type == "cuda" else 0
+        self._workgroup_slots_per_xcd = 2 * max(1, cus // 8)
         # the merged projection weights exist before the cache is sized from free device memory
         if self.device.type == "cuda" and hasattr(self.base_model, "model"):
             with torch.no_grad():
@@ -90,6 +94,10 @@ class ModelRunner:
 
     def _attention_modules(self):
         return [m for m in self.model.modules() if hasattr(m, "k_cache") and hasattr(m, "v_cache")]
+
+    def _attention_head_counts(self):
+        first = self._attention_modules()[0]
+        return first.num_heads, first.num_kv_heads
 
     # ------------------------------------------------------------------ timing (model_runner.py:80-140)
     def _profile_timing_enabled(self):
@@ -313,6 +321,27 @@ class ModelRunner:
         if self.device.type == "cuda":
             t = t.pin_memory()
         return t.to(self.device, non_blocking=True)
+
+    def _attention_plan(self, cu_q, cu_k):
+        """Dispatch plan of the attention kernel for a refresh forward with these prefix sums (host values), or
+        None where the order cannot matter: every layer of the forward shares it, and the refreshes of one batch
+        repeat the same lengths, so the last few plans are kept."""
+        if self.device.type != "cuda":
+            return None
+        cu_q, cu_k = np.asarray(cu_q, dtype=np.int32), np.asarray(cu_k, dtype=np.int32)
+        heads, kv_heads = self._attention_head_counts()
+        tiles = int(((np.diff(cu_q) + 127) // 128).sum())
+        slots = self._workgroup_slots_per_xcd
+        if tiles * heads <= 8 * slots:      # every unit starts at once
+            return None
+        key = (cu_q.tobytes(), cu_k.tobytes())
+        plan = self._attention_plans.pop(key, None)
+        if plan is None:
+            plan = ops.attention_plan(cu_q, cu_k, heads, kv_heads, self.device, slots)
+            if len(self._attention_plans) >= 8:
+                self._attention_plans.pop(next(iter(self._attention_plans)))
+        self._attention_plans[key] = plan   # most recently used last
+        return plan
 
     def _precompute_shared_prefix(self, prefix_tokens: list[int]):
         """One forward of the affix alone at positions ``0..A-1``; its post-RoPE K/V land in slots ``0..A-1``."""
@@ -742,7 +771,8 @@ class ModelRunner:
         current = np.array([s.current_block_idx for s in group])
         cu_dev = self._to_device(cu, torch.int32)
         set_context(True, cu_dev, cu_dev, None, int(lens.max()), int(lens.max()),
-                    self._to_device(slot_mapping, torch.int32), block_tables, total_k=int(cu[-1]))
+                    self._to_device(slot_mapping, torch.int32), block_tables, total_k=int(cu[-1]),
+                    attention_plan=self._attention_plan(cu, cu))
         return (self._to_device(input_ids, torch.int64), self._to_device(positions, torch.int64),
                 self._to_device(generate_starts, torch.int32), self._to_device(current, torch.int32))
 
@@ -795,7 +825,7 @@ class ModelRunner:
             self._to_device(np.concatenate(reads), torch.int32),
             self._to_device(shared_lens, torch.int32) if use_query_relocation else None,
             None if relocation_materialized else self._to_device(shifts, torch.int32),
-            total_k=int(cu_k[-1]))
+            total_k=int(cu_k[-1]), attention_plan=self._attention_plan(cu_q, cu_k))
         return (self._to_device(np.concatenate(ids), torch.int64), self._to_device(np.concatenate(pos), torch.int64),
                 self._to_device(block_starts, torch.int32))
 
@@ -842,7 +872,8 @@ class ModelRunner:
         set_context(
             True, d_cu_q, d_cu_k, d_kv, int(max(n_rec)), int(kv_lens.max()),
             torch.cat([l.recompute_slots for l in layouts]), None, True, torch.cat(reads),
-            d_shared if packed else None, d_shifts, total_k=int(cu_k[-1]))
+            d_shared if packed else None, d_shifts, total_k=int(cu_k[-1]),
+            attention_plan=self._attention_plan(cu_q, cu_k))
         return input_ids, positions, d_starts
 
     def _prepare_decoding_from_device_layouts(self, group):

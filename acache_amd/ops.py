@@ -558,8 +558,38 @@ def block_table_slots(
     return out
 
 
+def attention_plan(cu_seqlens_q, cu_seqlens_k, num_heads: int, num_kv_heads: int, device,
+                   slots_per_xcd: int | None = None) -> torch.Tensor:
+    """Dispatch plan for :func:`acache_attention` calls over these lengths: ``[blocks, 2]`` int32 on ``device``.
+
+    The prefix sums are read on the host (lists or CPU tensors cost nothing; device tensors are copied back,
+    which synchronises).  The plan depends only on the lengths and head counts, so one plan serves every layer
+    of a forward pass.  It orders the (request, query tile, head) units so that the hardware's in-order hand-out
+    of workgroups packs each XCD's slots tightly; results are bit-identical with and without it.  No counterpart
+    in the reference, whose Triton grid is (query block, head, request) in launch order (acache_attention.py:721).
+    """
+    cq = torch.as_tensor(cu_seqlens_q, dtype=torch.int32, device="cpu").contiguous()
+    ck = torch.as_tensor(cu_seqlens_k, dtype=torch.int32, device="cpu").contiguous()
+    assert cq.numel() == ck.numel() and cq.numel() >= 1
+    B = cq.numel() - 1
+    device = torch.device(device)
+    if slots_per_xcd is None:
+        slots_per_xcd = max(1, torch.cuda.get_device_properties(device).multi_processor_count // 8) * 2
+    lib = _lib.load()
+    args = (cq.data_ptr(), ck.data_ptr(), B, int(num_heads), int(num_kv_heads), int(slots_per_xcd))
+    blocks = lib.acache_varlen_attn_plan(*args, None, 0)
+    if blocks < 0:
+        _lib.check(int(blocks), "attention_plan")
+    plan = torch.empty(max(int(blocks), 0), 2, dtype=torch.int32, pin_memory=device.type == "cuda")
+    if blocks > 0:
+        rc = lib.acache_varlen_attn_plan(*args, plan.data_ptr(), int(blocks))
+        if rc < 0:
+            _lib.check(int(rc), "attention_plan")
+    return plan.to(device, non_blocking=True)
+
+
 def _varlen_attn(q, k_cache, v_cache, cu_q, cu_k, slots, scale, shared_prefix_len,
-                 shared_kv_lens, affix_shifts, cos, sin):
+                 shared_kv_lens, affix_shifts, cos, sin, plan=None):
     total_q, H, D = q.shape
     Hkv = k_cache.shape[-2]
     assert k_cache.shape[-1] == D and v_cache.shape == k_cache.shape
@@ -577,13 +607,21 @@ def _varlen_attn(q, k_cache, v_cache, cu_q, cu_k, slots, scale, shared_prefix_le
     B = cu_q.numel() - 1
     rope_rows = 0 if cos is None else cos.shape[0]
     lib = _lib.load()
+    plan_blocks = 0
+    if plan is not None:
+        assert plan.is_cuda and plan.dtype == torch.int32 and plan.dim() == 2 and plan.shape[1] == 2
+        assert plan.is_contiguous()
+        plan_blocks = plan.shape[0]
+        if plan_blocks == 0:
+            plan = None
     with torch.cuda.device(q.device):
-        rc = lib.acache_varlen_attn(
+        rc = lib.acache_varlen_attn_planned(
             _ptr(out), _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(cu_q), _ptr(cu_k), _ptr(slots),
             float(scale), int(shared_prefix_len), _ptr(shared_kv_lens), _ptr(affix_shifts),
             _ptr(cos), _ptr(sin), rope_rows,
             B, total_q, slots.numel(), H, Hkv, D, _code(q), num_slots,
-            q.stride(0), q.stride(1), out.stride(0), out.stride(1), slot_stride, head_stride, _stream(q))
+            q.stride(0), q.stride(1), out.stride(0), out.stride(1), slot_stride, head_stride,
+            _ptr(plan), plan_blocks, _stream(q))
     _lib.check(rc, "acache_attention")
     return out
 
@@ -601,11 +639,14 @@ def acache_attention(
     affix_shifts: torch.Tensor | None = None,
     rope_cos: torch.Tensor | None = None,
     rope_sin: torch.Tensor | None = None,
+    plan: torch.Tensor | None = None,
 ):
     """Bidirectional varlen attention over K/V read through ``read_slot_mapping``.
 
     Argument order, mode selection and ``ValueError`` conditions follow the
-    reference wrapper (acache_attention.py:643-738).  Differences: no host
+    reference wrapper (acache_attention.py:643-738); ``plan`` (from :func:`attention_plan`
+    for the same lengths) is an addition that only changes the order the units run in.
+    Differences: no host
     synchronisation (the reference reads ``max_q`` and the table-size check back
     with ``.item()``, lines 667 and 685); a key whose shift exceeds the table is
     left unrotated instead of reading out of bounds; rows of requests without
@@ -639,7 +680,7 @@ def acache_attention(
     return _varlen_attn(
         q, k_cache, v_cache, _i32(cu_seqlens_q, "cu_seqlens_q"), _i32(cu_seqlens_k, "cu_seqlens_k"),
         _i32(read_slot_mapping, "read_slot_mapping"), softmax_scale,
-        shared_prefix_len if apply_relocation else 0, shared, shifts, cos, sin)
+        shared_prefix_len if apply_relocation else 0, shared, shifts, cos, sin, plan)
 
 
 def baseline_ragged_attention(
@@ -651,6 +692,7 @@ def baseline_ragged_attention(
     block_tables: torch.Tensor,
     softmax_scale: float | None = None,
     total_k: int | None = None,
+    plan: torch.Tensor | None = None,
 ):
     """Varlen attention over block-table paged K/V (full-recompute baseline).
 
@@ -667,7 +709,7 @@ def baseline_ragged_attention(
     cu_k = _i32(cu_seqlens_k, "cu_seqlens_k")
     slots = block_table_slots(block_tables, cu_k, k_cache.shape[1], total_k)
     return _varlen_attn(q, k_cache, v_cache, _i32(cu_seqlens_q, "cu_seqlens_q"), cu_k, slots,
-                        softmax_scale, 0, None, None, None, None)
+                        softmax_scale, 0, None, None, None, None, plan)
 
 
 def baseline_decode_attention(

@@ -159,14 +159,29 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
     vc = (torch.randn(w["num_blocks"], BS, Hkv, D, generator=gen, device=device) / D ** 0.5).to(torch.bfloat16)
     cu_q, cu_k, slots = w["cu_q"].to(device), w["cu_k"].to(device), w["slot_map"].to(device)
 
-    def step():
-        return ops.acache_attention(q, kc, vc, cu_q, cu_k, slots)
+    # the dispatch plan of these lengths, made on the host once as the engine makes it once per forward pass for
+    # all of its layers; the call without a plan (units ordered inside the kernel) is timed next to it
+    t0 = time.perf_counter()
+    plan = ops.attention_plan(w["cu_q"], w["cu_k"], H, Hkv, device)
+    plan_host_ms = (time.perf_counter() - t0) * 1e3
 
-    for _ in range(warmup):
+    def step():
+        return ops.acache_attention(q, kc, vc, cu_q, cu_k, slots, plan=plan)
+
+    # A launch takes about 0.1 ms: a region of 20 launches is 2 ms long and carries the idle time in front of its
+    # first launch (about 5 us per launch), and three launches after the CPU legs do not bring the clocks back up.
+    # The leg therefore times at least 200 launches after at least 50 untimed ones and says so in its line.
+    attn_warmup, attn_steps = max(warmup, 50), max(steps, 200)
+    for _ in range(attn_warmup):
         step()
     torch.cuda.synchronize()
-    ms = _event_times_ms(step, steps, torch)
+    ms = _event_times_ms(step, attn_steps, torch)
     avg_ms = sum(ms) / len(ms)
+    for _ in range(attn_warmup):
+        ops.acache_attention(q, kc, vc, cu_q, cu_k, slots)
+    torch.cuda.synchronize()
+    unplanned_ms = _event_times_ms(lambda: ops.acache_attention(q, kc, vc, cu_q, cu_k, slots), attn_steps, torch)
+    unplanned_ms = sum(unplanned_ms) / len(unplanned_ms)
     flops = 4 * H * D * sum(a * b for a, b in zip(w["q_lens"], w["kv_lens"]))
     kv_bytes = 2 * sum(w["kv_lens"]) * Hkv * D * 2
     qo_bytes = 2 * total_q * H * D * 2
@@ -201,8 +216,11 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
         **extra,
         "metric": "anchor-recompute attn TFLOP/s", "value": round(tflops, 1), "unit": "TFLOP/s",
         "ms_per_call": round(avg_ms, 4),
+        "ms_per_call_without_plan": round(unplanned_ms, 4), "plan_host_ms": round(plan_host_ms, 3),
+        "launches_timed": attn_steps, "warmup_launches": attn_warmup,
         "config": {"workload": "configs[3]: batch 16, 32 heads (MHA), D 128, bf16, q = 20% anchors + 32 per request, "
-                               "kv = affix + request + 256 (920-1712), slot map over shared affix slots and shuffled private blocks",
+                               "kv = affix + request + 256 (920-1712), slot map over shared affix slots and shuffled private "
+                               "blocks; units dispatched by a host-made plan of the lengths (made once, outside the timed calls)",
                    "total_q": total_q, "total_kv": sum(w["kv_lens"])},
         "roofline": {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES["attention"],

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define ACACHE_ABI_VERSION 3
+#define ACACHE_ABI_VERSION 4
 
 /* element types of K/V/Q payloads */
 #define ACACHE_BF16 0
@@ -363,6 +363,19 @@ int acache_build_slot_layout(
  * unit, two workgroups per CU, units handed out longest request first; K/V tiles of 64 keys reach LDS
  * through the copy engine.  In key-side mode the rows of a tile that lie in shared slots are re-rotated
  * in LDS after they land.  No workspace: the kernel allocates nothing and keeps no state between calls.
+ *
+ * acache_varlen_attn_planned is the same call with the order of the units given by the caller:
+ * `plan` (device memory, 8-byte aligned, 2 * plan_blocks int32, written by
+ * acache_varlen_attn_plan for the same cu_q, cu_k, H and H_kv) names the unit of every block of the
+ * grid.  The hardware hands blocks out in index order, so with two or three units per workgroup
+ * slot the order decides how evenly the slots finish; a plan packs them (measured on configs[3] of
+ * the benchmark: 96 -> 87 us).  Results are bit-identical with and without a plan.  The kernel checks
+ * every plan entry against B, H and cu_q: a plan made for other lengths can leave output rows
+ * unwritten, it cannot cause an access outside the call's buffers.  plan == NULL is
+ * acache_varlen_attn; head_dim other than 64 / 128 ignores the plan.  One plan serves every layer
+ * of a forward pass (it depends on the lengths and head counts only).  No counterpart in the
+ * reference, whose Triton grid is (query block, head, request) in launch order
+ * (acache_attention.py:721-737).
  */
 int acache_varlen_attn(
     void *out, const void *q, const void *k_cache, const void *v_cache,
@@ -375,6 +388,38 @@ int acache_varlen_attn(
     int64_t q_token_stride, int64_t q_head_stride,
     int64_t out_token_stride, int64_t out_head_stride,
     int64_t kv_slot_stride, int64_t kv_head_stride, void *stream);
+
+int acache_varlen_attn_planned(
+    void *out, const void *q, const void *k_cache, const void *v_cache,
+    const int32_t *cu_q, const int32_t *cu_k, const int32_t *slot_map,
+    float scale,
+    int32_t shared_prefix_len, const int32_t *shared_kv_lens, const int32_t *affix_shifts,
+    const float *rope_cos, const float *rope_sin, int32_t rope_rows,
+    int32_t B, int64_t total_q, int64_t total_k,
+    int32_t H, int32_t H_kv, int32_t D, int32_t dtype, int64_t num_slots,
+    int64_t q_token_stride, int64_t q_head_stride,
+    int64_t out_token_stride, int64_t out_head_stride,
+    int64_t kv_slot_stride, int64_t kv_head_stride,
+    const int32_t *plan, int64_t plan_blocks, void *stream);
+
+/*
+ * Host-side planner of acache_varlen_attn_planned: no GPU work, no device pointers.
+ * cu_q_host / cu_k_host are HOST copies of the call's prefix sums (B + 1 entries each).
+ * Returns the number of blocks of the plan (a multiple of 8, >= 0) or an ACACHE_E_* code.
+ * With plan_host == NULL only the size is computed; otherwise 2 * blocks int32 are written
+ * (capacity_blocks must be at least the returned size), to be copied to the device by the
+ * caller.  Entry i is (request, tile | head << 20) for block i, request -1 = no work.
+ * slots_per_xcd = workgroups of the attention kernel that one XCD holds at a time
+ * (2 * CUs / 8; <= 0 selects 64, the MI355X value).  Every unit stays on the XCD that shares
+ * its KV head's rows in L2; per XCD the units are packed into `slots_per_xcd` bins by a cost
+ * model (a fixed part plus a term per 64-key tile, cheaper for tiles of at most 64 / 32 live
+ * rows) and issued in the order of their start times in that packing.  Lists of at most one
+ * unit per slot or of more than 16 per slot are issued longest first.  Host cost: about
+ * 0.1 ms for a batch of 16 requests and 32 heads.
+ */
+int64_t acache_varlen_attn_plan(
+    const int32_t *cu_q_host, const int32_t *cu_k_host, int32_t B, int32_t H, int32_t H_kv,
+    int32_t slots_per_xcd, int32_t *plan_host, int64_t capacity_blocks);
 
 /*
  * Two elementwise steps of the decoder block on either side of the attention path, for

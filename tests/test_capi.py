@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in _declared_functions():
         assert hasattr(lib, name), name
-    assert lib.acache_abi_version() == 3
+    assert lib.acache_abi_version() == 4
 
 
 def test_argument_errors_are_reported_without_a_device():

@@ -480,3 +480,45 @@ def test_request_longer_than_the_configured_length_is_served(device):
     got, nfe = run(model, cfg)
     want, nfe_want = run(wide, wide_cfg)
     assert got == want and nfe == nfe_want and 63 not in got[0]
+
+
+@pytest.mark.parametrize("use_acache", [True, False])
+def test_refresh_forwards_run_under_a_dispatch_plan_and_give_the_same_tokens(device, use_acache):
+    """With more attention units than workgroup slots a refresh forward carries a dispatch plan in its context
+    (one per distinct set of lengths, reused by later refreshes); the generated tokens equal those of a runner
+    that never plans."""
+    cfg, model = _model(device, seed=1)
+    affix = list(range(20, 30))
+
+    def make(i):
+        toks = [2 + i] + affix + [40 + i, 41 + i]
+        return Sequence(toks, gen_length=8, block_length=4, cache_block_size=8, mask_id=63,
+                        prompt_affix_start=1, prompt_affix_end=11)
+
+    def generate(plans):
+        serve = _serve(cfg, recompute_batch_size=2, max_num_seqs=0, gen_length=8, block_length=4,
+                       num_kvcache_blocks=32, threshold=0.9, anchor_ratio=0.5, enable_acache=use_acache)
+        runner = ModelRunner(model, serve)
+        seen = []
+        if plans:
+            runner._workgroup_slots_per_xcd = 0        # any number of units counts as more than the slots
+            real = runner._attention_plan
+
+            def spy(cu_q, cu_k):
+                plan = real(cu_q, cu_k)
+                seen.append(plan)
+                return plan
+
+            runner._attention_plan = spy
+        else:
+            runner._attention_plan = lambda cu_q, cu_k: None
+        seqs = [make(i) for i in range(4)]
+        out, _ = runner.generate_with_acache(seqs) if use_acache else runner.generate_with_dual_cache(seqs)
+        return out, seen, runner
+
+    planned, seen, runner = generate(True)
+    assert seen and all(p is not None and p.shape[0] % 8 == 0 and p.shape[0] > 0 for p in seen)
+    assert len({p.data_ptr() for p in seen}) < len(seen)      # later refreshes of the same lengths reuse a plan
+    assert len(runner._attention_plans) <= 8
+    unplanned, _, _ = generate(False)
+    assert planned == unplanned
