@@ -160,7 +160,7 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
     cu_q, cu_k, slots = w["cu_q"].to(device), w["cu_k"].to(device), w["slot_map"].to(device)
 
     # the dispatch plan of these lengths, made on the host once as the engine makes it once per forward pass for
-    # all of its layers; the call without a plan (units ordered inside the kernel) is timed next to it
+    # all of its layers (`--attention-shapes` times the same call with and without a plan)
     t0 = time.perf_counter()
     plan = ops.attention_plan(w["cu_q"], w["cu_k"], H, Hkv, device)
     plan_host_ms = (time.perf_counter() - t0) * 1e3
@@ -177,11 +177,6 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
     torch.cuda.synchronize()
     ms = _event_times_ms(step, attn_steps, torch)
     avg_ms = sum(ms) / len(ms)
-    for _ in range(attn_warmup):
-        ops.acache_attention(q, kc, vc, cu_q, cu_k, slots)
-    torch.cuda.synchronize()
-    unplanned_ms = _event_times_ms(lambda: ops.acache_attention(q, kc, vc, cu_q, cu_k, slots), attn_steps, torch)
-    unplanned_ms = sum(unplanned_ms) / len(unplanned_ms)
     flops = 4 * H * D * sum(a * b for a, b in zip(w["q_lens"], w["kv_lens"]))
     kv_bytes = 2 * sum(w["kv_lens"]) * Hkv * D * 2
     qo_bytes = 2 * total_q * H * D * 2
@@ -216,7 +211,7 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
         **extra,
         "metric": "anchor-recompute attn TFLOP/s", "value": round(tflops, 1), "unit": "TFLOP/s",
         "ms_per_call": round(avg_ms, 4),
-        "ms_per_call_without_plan": round(unplanned_ms, 4), "plan_host_ms": round(plan_host_ms, 3),
+        "plan_host_ms": round(plan_host_ms, 3),
         "launches_timed": attn_steps, "warmup_launches": attn_warmup,
         "config": {"workload": "configs[3]: batch 16, 32 heads (MHA), D 128, bf16, q = 20% anchors + 32 per request, "
                                "kv = affix + request + 256 (920-1712), slot map over shared affix slots and shuffled private "
@@ -477,8 +472,27 @@ def attention_shape_sweep(torch, device, ops, steps):
             call()
         ms = _event_times_ms(call, steps, torch)[0]
         modes.append({"mode": name, "us": round(ms * 1e3, 1), "TFLOPs": round(flops / ms / 1e9, 0)})
+    # The benchmark's anchor-recompute batch (configs[3]) with the units ordered inside the kernel (longest request
+    # first) and under a host-made dispatch plan; MHA as the benchmark runs it and with 8 KV heads.
+    from acache_amd.synthetic import attention_batch
+    w = attention_batch(seed=0)
+    plan_rows = []
+    for H, Hkv in ((32, 32), (32, 8)):
+        Q = (torch.randn(int(w["cu_q"][-1]), H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        K = (torch.randn(w["num_blocks"], 256, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        V = (torch.randn(w["num_blocks"], 256, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        cu_q, cu_k, slots = w["cu_q"].to(device), w["cu_k"].to(device), w["slot_map"].to(device)
+        plan = ops.attention_plan(w["cu_q"], w["cu_k"], H, Hkv, device)
+        row = {"H": H, "H_kv": Hkv}
+        for name, p in (("in_kernel_order_us", None), ("planned_us", plan), ("in_kernel_order_again_us", None),
+                        ("planned_again_us", plan)):
+            call = lambda: ops.acache_attention(Q, K, V, cu_q, cu_k, slots, plan=p)
+            for _ in range(50):
+                call()
+            row[name] = round(_event_times_ms(call, max(steps, 200), torch)[0] * 1e3, 1)
+        plan_rows.append(row)
     print(json.dumps({"attention_shape_sweep": rows, "decode_shapes_with_shared_affix_rows": shared_rows,
-                      "relocation_modes": modes}))
+                      "relocation_modes": modes, "anchor_recompute_batch_dispatch_plan": plan_rows}))
 
 
 def kernel_sweep(torch, device, ops, steps):
