@@ -26,7 +26,10 @@ struct ScatterParams {
   int32_t L;
 };
 
-template <int LPB>
+// STREAM: non-temporal stores.  A launch that writes more than the L2 holds gains 13 % from them (68 -> 59 us
+// for 166 MB of rows into shuffled blocks); a small one keeps ordinary stores, so that the attention call
+// behind it finds the fresh rows in L2.
+template <int LPB, bool STREAM>
 __global__ __launch_bounds__(256) void scatter_kernel(ScatterParams p) {
   const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t token = gid / p.chunks_per_token;
@@ -49,8 +52,10 @@ __global__ __launch_bounds__(256) void scatter_kernel(ScatterParams p) {
 #pragma unroll
   for (int i = 0; i < LPB; ++i) {
     if (l0 + i < p.L) {
-      store16(p.k_cache + (int64_t)(l0 + i) * p.cache_layer_bytes + dst, k[i]);
-      store16(p.v_cache + (int64_t)(l0 + i) * p.cache_layer_bytes + dst, v[i]);
+      char *const kd = p.k_cache + (int64_t)(l0 + i) * p.cache_layer_bytes + dst;
+      char *const vd = p.v_cache + (int64_t)(l0 + i) * p.cache_layer_bytes + dst;
+      if (STREAM) { store16_stream(kd, k[i]); store16_stream(vd, v[i]); }
+      else { store16(kd, k[i]); store16(vd, v[i]); }
     }
   }
 }
@@ -167,7 +172,10 @@ extern "C" int acache_kv_scatter(
   constexpr int LPB = 2;
   if (gx > 0x7fffffffLL || (L + LPB - 1) / LPB > 65535) return fail(ACACHE_E_SHAPE, "kv_scatter: too many rows or layers");
   dim3 grid((unsigned)gx, (unsigned)((L + LPB - 1) / LPB));
-  hipLaunchKernelGGL(scatter_kernel<LPB>, grid, dim3(256), 0, (hipStream_t)stream, p);
+  // rows written by one launch, K and V: beyond 32 MiB (eight times the 4 MiB L2 of an XCD) they stream
+  const bool stream_stores = N * tok * es * 2 * L > (32LL << 20);
+  if (stream_stores) hipLaunchKernelGGL((scatter_kernel<LPB, true>), grid, dim3(256), 0, (hipStream_t)stream, p);
+  else hipLaunchKernelGGL((scatter_kernel<LPB, false>), grid, dim3(256), 0, (hipStream_t)stream, p);
   return launch_status("scatter_kernel");
 }
 
