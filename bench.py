@@ -169,9 +169,11 @@ def attention_bench(torch, device, ops, steps, warmup, cpu_baseline=False):
         return ops.acache_attention(q, kc, vc, cu_q, cu_k, slots, plan=plan)
 
     # A launch takes about 0.1 ms: a region of 20 launches is 2 ms long and carries the idle time in front of its
-    # first launch (about 5 us per launch), and three launches after the CPU legs do not bring the clocks back up.
-    # The leg therefore times at least 200 launches after at least 50 untimed ones and says so in its line.
-    attn_warmup, attn_steps = max(warmup, 50), max(steps, 200)
+    # first launch (about 5 us per launch), and after the CPU legs the chip needs about 270 launches (27 ms) to
+    # come back to the clocks it holds under load (regions of 200 launches after an idle period measure 100, 95.2,
+    # 95.7, 95.6 us per launch).  The leg therefore times at least 200 launches after at least 300 untimed ones
+    # and says so in its line.
+    attn_warmup, attn_steps = max(warmup, 300), max(steps, 200)
     for _ in range(attn_warmup):
         step()
     torch.cuda.synchronize()
