@@ -65,6 +65,14 @@ def test_planned_call_gives_the_bits_of_the_unplanned_one(device, mode, H, Hkv, 
         assert torch.equal(_run(t, kw, device, plan), _run(t, kw, device))
 
 
+@pytest.mark.parametrize("B", [70, 150])
+def test_more_than_64_requests(device, B):
+    """Above 64 requests the unplanned kernel walks the requests in batch order; a plan orders any batch."""
+    t, kw = _batch(B, B, 8, 8, 128, torch.bfloat16, "query", device, A=64)
+    plan = ops.attention_plan(t["cu_q"], t["cu_k"], 8, 8, device)
+    assert torch.equal(_run(t, kw, device, plan), _run(t, kw, device))
+
+
 def test_planned_call_against_the_oracle(device):
     t, kw = _batch(5, 6, 4, 2, 128, torch.bfloat16, "key", device)
     plan = ops.attention_plan(t["cu_q"], t["cu_k"], 4, 2, device, slots_per_xcd=2)
