@@ -388,8 +388,9 @@ def reference_generate_partial(model, prompt, a0, A, ratio, steps, gen_length, b
     return x, nfe, anchors.tolist(), min(margins)
 
 
+@pytest.mark.parametrize("threshold", [None, 0.03], ids=["quota", "threshold"])
 @pytest.mark.parametrize("placement", ["prefix", "infix"])
-def test_partial_ratio_generation_equals_the_restated_loop(device, placement):
+def test_partial_ratio_generation_equals_the_restated_loop(device, placement, threshold):
     """Anchor ratio 0.25: importance pass, top-k anchors, frozen non-anchor affix rows, recompute of anchors and
     non-affix tokens at every block boundary.  Tokens and forward count must equal the restated reference loop, with
     the engine's own affix precompute and with the affix cache in Dream's layout handed in."""
@@ -403,18 +404,19 @@ def test_partial_ratio_generation_equals_the_restated_loop(device, placement):
         sd = _checkpoint_state(seed)
         ref = TorchDream(sd)
         want, nfe_want, anchors, margin = reference_generate_partial(ref, prompt, a0, A, 0.25, steps=8, gen_length=8,
-                                                                    block_length=4)
+                                                                    block_length=4, threshold=threshold)
         if margin > 1.0 and len(set(want[-8:].tolist())) >= 4:            # decisive and not one token eight times
             break
     else:
         pytest.fail("no seed with comfortable decision margins")
     assert len(anchors) == 6 and (want != MASK).all()
     # the frozen affix rows matter: recomputing the whole affix (every token an anchor) decodes other tokens
-    everything, _, _ = reference_generate(ref, prompt, steps=8, gen_length=8, block_length=4, threshold=None,
+    everything, _, _ = reference_generate(ref, prompt, steps=8, gen_length=8, block_length=4, threshold=threshold,
                                           generation_start=None)
     assert everything.tolist() != want.tolist()
     model = _engine_model(sd, device)
-    kw = dict(steps=8, gen_length=8, block_length=4, mask_id=MASK, anchor_ratio=0.25, affix_start=a0, affix_end=a0 + A)
+    kw = dict(steps=8, gen_length=8, block_length=4, mask_id=MASK, anchor_ratio=0.25, affix_start=a0, affix_end=a0 + A,
+              threshold=threshold)
     got, nfe = GD.generate_with_anchor_attention(model, torch.tensor([prompt], device=device), **kw)
     assert got[0].cpu().tolist() == want.tolist() and nfe == nfe_want
     # the same call with the reference-layout affix cache: [1, A, H_kv * D] per layer, keys before RoPE
