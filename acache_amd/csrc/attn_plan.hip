@@ -10,6 +10,7 @@
 //
 // Units of one KV head stay on the XCDs that share that head's rows in L2, as in the kernel's own index map.
 #include <algorithm>
+#include <exception>
 #include <numeric>
 #include <queue>
 #include <vector>
@@ -28,7 +29,7 @@ struct Unit {
 // epilogue) plus one term per key tile, cheaper when at most 64 / 32 query rows are live and two waves share
 // a row block.
 inline int32_t unit_cost(int rows, int kv_len) {
-  const int kt = (kv_len + 63) / 64;
+  const int kt = std::min(kv_len / 64 + (kv_len % 64 != 0), 1 << 20);  // beyond that only the order matters
   const int per_tile = rows > 64 ? 100 : (rows > 32 ? 85 : 60);
   return 290 + kt * per_tile;
 }
@@ -94,9 +95,8 @@ void plan_order(const std::vector<int32_t> &costs, int slots, std::vector<int32_
 
 using namespace acache;
 
-extern "C" int64_t acache_varlen_attn_plan(const int32_t *cu_q_host, const int32_t *cu_k_host, int32_t B, int32_t H,
-                                           int32_t H_kv, int32_t slots_per_xcd, int32_t *plan_host,
-                                           int64_t capacity_blocks) {
+static int64_t make_plan(const int32_t *cu_q_host, const int32_t *cu_k_host, int32_t B, int32_t H, int32_t H_kv,
+                         int32_t slots_per_xcd, int32_t *plan_host, int64_t capacity_blocks) {
   if (B < 0 || H <= 0 || H_kv <= 0 || H % H_kv != 0 || H >= (1 << 11))
     return fail(ACACHE_E_SHAPE, "varlen_attn_plan: bad sizes (B=%d, H=%d, H_kv=%d)", B, H, H_kv);
   if (B > 0 && (!cu_q_host || !cu_k_host)) return fail(ACACHE_E_NULL, "varlen_attn_plan: NULL pointer");
@@ -167,4 +167,14 @@ extern "C" int64_t acache_varlen_attn_plan(const int32_t *cu_q_host, const int32
     }
   }
   return blocks;
+}
+
+extern "C" int64_t acache_varlen_attn_plan(const int32_t *cu_q_host, const int32_t *cu_k_host, int32_t B, int32_t H,
+                                           int32_t H_kv, int32_t slots_per_xcd, int32_t *plan_host,
+                                           int64_t capacity_blocks) {
+  try {
+    return make_plan(cu_q_host, cu_k_host, B, H, H_kv, slots_per_xcd, plan_host, capacity_blocks);
+  } catch (const std::exception &e) {  // the planner's own vectors: nothing may unwind through the C boundary
+    return fail(ACACHE_E_SHAPE, "varlen_attn_plan: %s", e.what());
+  }
 }
