@@ -1037,8 +1037,7 @@ class ModelRunner:
                     current_blocks = working[part]
                     x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
                                                            current_blocks, threshold)
-                    r, c = torch.where(transfer)
-                    working[part[r], c] = x0[transfer]
+                    working[part] = torch.where(transfer, x0, current_blocks)   # no read-back of the picks
                 self._finish_timing(timing, "cache_update", start)
             total_nfe += len(rows)
 
@@ -1135,8 +1134,7 @@ class ModelRunner:
                 current_blocks = working[active]
                 x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
                                                        current_blocks, threshold)
-                r, c = torch.where(transfer)
-                working[active[r], c] = x0[transfer]
+                working[active] = torch.where(transfer, x0, current_blocks)       # no read-back of the picks
                 stalled = (working[active] == mask_id).sum() >= (current_blocks == mask_id).sum()
                 self._finish_timing(timing, "decode_update", start)
                 total_nfe += len(active)
@@ -1211,7 +1209,7 @@ class ModelRunner:
         committable = mask_index & (x0 != self.config.mask_id)
         confidence = torch.where(committable, x0_p, torch.full_like(x0_p, -math.inf))
         transfer = (confidence >= threshold) & committable
+        # a row with committable positions and none above the threshold commits its most confident one
         stuck = committable.any(dim=1) & ~transfer.any(dim=1)
-        rows = torch.where(stuck)[0]
-        transfer[rows, confidence.argmax(dim=1)[rows]] = True
-        return x0, transfer
+        forced = torch.zeros_like(transfer).scatter_(1, confidence.argmax(dim=1, keepdim=True), stuck.unsqueeze(1))
+        return x0, transfer | forced
