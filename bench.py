@@ -493,8 +493,41 @@ def attention_shape_sweep(torch, device, ops, steps):
                 call()
             row[name] = round(_event_times_ms(call, max(steps, 200), torch)[0] * 1e3, 1)
         plan_rows.append(row)
+    # The same comparison on other shapes the engine issues: a block refresh of four requests at anchor ratio 0.2
+    # (613 queries, 1 413 keys of which 800 are shared affix rows), a uniform batch, a refinement step.
+    def ragged_case(name, q_lens, kv_lens, H, Hkv, shared):
+        cu = lambda lens: torch.tensor([0] + torch.tensor(lens).cumsum(0).tolist(), dtype=torch.int32)
+        cu_q, cu_k = cu(q_lens), cu(kv_lens)
+        pieces, nxt = [], shared
+        for kv in kv_lens:
+            pieces += [torch.arange(shared), nxt + torch.arange(kv - shared)]
+            nxt += kv - shared
+        slots = torch.cat(pieces).to(torch.int32).to(device)
+        nb = (nxt + 255) // 256
+        Q = (torch.randn(int(cu_q[-1]), H, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        K = (torch.randn(nb, 256, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        V = (torch.randn(nb, 256, Hkv, D, device=device) / D ** 0.5).to(torch.bfloat16)
+        dq, dk = cu_q.to(device), cu_k.to(device)
+        plan = ops.attention_plan(cu_q, cu_k, H, Hkv, device)
+        row = {"shape": name, "H": H, "H_kv": Hkv, "units_per_xcd": plan.shape[0] // 8}
+        for key, p in (("in_kernel_order_us", None), ("planned_us", plan), ("in_kernel_order_again_us", None),
+                       ("planned_again_us", plan)):
+            call = lambda: ops.acache_attention(Q, K, V, dq, dk, slots, plan=p)
+            for _ in range(30):
+                call()
+            row[key] = round(_event_times_ms(call, max(steps, 100), torch)[0] * 1e3, 1)
+        return row
+
+    other_rows = [
+        ragged_case("block refresh, 4 requests, anchor ratio 0.2", [613, 600, 640, 590], [1413, 1400, 1440, 1390], 32, 32, 800),
+        ragged_case("block refresh, 4 requests, full recompute", [1413, 1400, 1440, 1390], [1413, 1400, 1440, 1390], 32, 32, 0),
+        ragged_case("uniform 16 x 600 x 1400", [600] * 16, [1400] * 16, 32, 32, 0),
+        ragged_case("Dream heads, 16 x 232 x 1400", [232] * 16, [1400] * 16, 28, 4, 1000),
+        ragged_case("refinement step, 16 x 32 x 1400", [32] * 16, [1400] * 16, 32, 32, 1000),
+    ]
     print(json.dumps({"attention_shape_sweep": rows, "decode_shapes_with_shared_affix_rows": shared_rows,
-                      "relocation_modes": modes, "anchor_recompute_batch_dispatch_plan": plan_rows}))
+                      "relocation_modes": modes, "anchor_recompute_batch_dispatch_plan": plan_rows,
+                      "dispatch_plan_other_shapes": other_rows}))
 
 
 def kernel_sweep(torch, device, ops, steps):
