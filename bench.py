@@ -44,7 +44,7 @@ MEASURED_TRAFFIC = {
                           "sources": ["acache_amd/csrc/scatter.hip", "acache_amd/csrc/common.h"]},
     "attention": {"bytes": 349.8e6, "commit": "b3bc566",
                   "sources": ["acache_amd/csrc/attn.hip", "acache_amd/csrc/attn_common.h", "acache_amd/csrc/mma.h",
-                              "acache_amd/csrc/common.h"]},
+                              "acache_amd/csrc/common.h", "acache_amd/csrc/attn_plan.hip"]},
 }
 MEASURED_TRAFFIC_BYTES = {name: entry["bytes"] for name, entry in MEASURED_TRAFFIC.items()}
 MEASURED_TRAFFIC_COMMIT = ", ".join(f"{name}: {entry['commit']}" for name, entry in MEASURED_TRAFFIC.items())
