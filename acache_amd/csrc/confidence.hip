@@ -127,6 +127,61 @@ __global__ __launch_bounds__(kConfThreads) void confidence_kernel(ConfidencePara
 
 using namespace acache;
 
+// The commit rule of block-wise decoding on one row of a block per wave: among the positions that still hold the
+// mask token and whose proposal is another token, commit the proposals whose confidence reaches the threshold, and
+// when there are such positions but none reaches it, the most confident one (the first of equals).  Positions are
+// walked twice (decide, then write); a row is 32 to a few hundred positions.
+__global__ __launch_bounds__(64) void commit_tokens_kernel(int64_t *blocks, const int64_t *proposal, const float *conf,
+                                                           int32_t *committed_rows, int L, int64_t mask_id,
+                                                           float threshold) {
+  const int lane = threadIdx.x;
+  int64_t *row = blocks + (int64_t)blockIdx.x * L;
+  const int64_t *prop = proposal + (int64_t)blockIdx.x * L;
+  const float *cf = conf + (int64_t)blockIdx.x * L;
+  bool any_committable = false, any_above = false;
+  float best = -INFINITY;
+  int best_at = 0x7fffffff;
+  for (int i = lane; i < L; i += 64) {
+    const bool committable = row[i] == mask_id && prop[i] != mask_id;
+    if (!committable) continue;
+    const float c = cf[i];
+    any_committable = true;
+    any_above |= c >= threshold;
+    if (c > best || best_at == 0x7fffffff) { best = c; best_at = i; }  // i ascends: the first of equals stays
+  }
+  const bool row_committable = __builtin_amdgcn_ballot_w64(any_committable) != 0;
+  const bool row_above = __builtin_amdgcn_ballot_w64(any_above) != 0;
+  if (!row_committable) return;
+  int forced = -1;
+  if (!row_above) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const float ob = __shfl_xor(best, d);
+      const int oa = __shfl_xor(best_at, d);
+      if (oa != 0x7fffffff && (best_at == 0x7fffffff || ob > best || (ob == best && oa < best_at))) { best = ob; best_at = oa; }
+    }
+    forced = best_at;
+  }
+  for (int i = lane; i < L; i += 64) {
+    const int64_t tok = prop[i];
+    const bool committable = row[i] == mask_id && tok != mask_id;
+    if (committable && (i == forced || (row_above && cf[i] >= threshold))) row[i] = tok;
+  }
+  if (lane == 0) atomicAdd(committed_rows, 1);
+}
+
+extern "C" int acache_commit_tokens(int64_t *blocks, const int64_t *proposal, const float *confidence,
+                                    int32_t *committed_rows, int64_t n, int32_t L, int64_t mask_id, float threshold,
+                                    void *stream) {
+  if (n < 0 || L <= 0) return fail(ACACHE_E_SHAPE, "commit_tokens: n %lld, L %d", (long long)n, L);
+  if (n == 0) return 0;
+  if (!blocks || !proposal || !confidence || !committed_rows) return fail(ACACHE_E_NULL, "commit_tokens: NULL pointer");
+  if (n > 0x7fffffffLL) return fail(ACACHE_E_SHAPE, "commit_tokens: too many rows");
+  hipLaunchKernelGGL(commit_tokens_kernel, dim3((unsigned)n), dim3(64), 0, (hipStream_t)stream, blocks, proposal,
+                     confidence, committed_rows, L, mask_id, threshold);
+  return launch_status("commit_tokens_kernel");
+}
+
 extern "C" int acache_argmax_confidence(
     int64_t *out_token, float *out_conf, const void *logits, const int64_t *picks,
     int64_t R, int64_t V, int64_t row_stride, int32_t dtype, void *stream) {

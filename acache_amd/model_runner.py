@@ -999,6 +999,7 @@ class ModelRunner:
             raise RuntimeError(f"No requests could be admitted under the current {budget}.")
         working = torch.full((batch_size, block_length), mask_id, dtype=torch.int64, device=device)
         offsets = torch.arange(block_length, device=device)
+        committed_rows = torch.zeros(1, dtype=torch.int32, device=device)   # rows that committed a token in a step
 
         def refresh(rows: torch.Tensor):
             """Cache refresh of the listed batch rows, ``recompute_batch_size`` requests per forward."""
@@ -1034,10 +1035,8 @@ class ModelRunner:
                     # a refresh commits only the first token of the block (model_runner.py:68-78, 1548-1552)
                     working[part, 0] = self._sample_dream_seed_tokens(logits[:, 0])
                 else:
-                    current_blocks = working[part]
-                    x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
-                                                           current_blocks, threshold)
-                    working[part] = torch.where(transfer, x0, current_blocks)   # no read-back of the picks
+                    working[part] = self._commit_from_logits(logits, working[part], temperature, remasking, threshold,
+                                                             committed_rows)
                 self._finish_timing(timing, "cache_update", start)
             total_nfe += len(rows)
 
@@ -1131,11 +1130,10 @@ class ModelRunner:
                 self._add_timing_count(timing, "decode_forward_nfe", len(active))
                 self._add_timing_count(timing, "decode_forward_tokens", len(active) * block_length)
                 start = self._start_timing()
-                current_blocks = working[active]
-                x0, transfer = self.get_transfer_index(logits, temperature, remasking, current_blocks == mask_id,
-                                                       current_blocks, threshold)
-                working[active] = torch.where(transfer, x0, current_blocks)       # no read-back of the picks
-                stalled = (working[active] == mask_id).sum() >= (current_blocks == mask_id).sum()
+                committed_rows.zero_()
+                working[active] = self._commit_from_logits(logits, working[active], temperature, remasking, threshold,
+                                                           committed_rows)
+                stalled = committed_rows == 0     # read at the top of the loop
                 self._finish_timing(timing, "decode_update", start)
                 total_nfe += len(active)
 
@@ -1175,6 +1173,27 @@ class ModelRunner:
         return logits.argmax(dim=-1)
 
     # ------------------------------------------------------------------ token transfer (2279-2314)
+    def _commit_from_logits(self, logits, current_blocks, temperature, remasking, threshold, committed_rows):
+        """``current_blocks`` with this step's picks written in, by the rule of ``get_transfer_index``.  With
+        confidence-based remasking and logits the confidence kernel takes, proposal, confidence and commit are
+        two or three launches; otherwise the tensor formulation.  ``committed_rows`` counts rows that committed."""
+        fused = (remasking == "low_confidence" and logits.is_cuda and logits.is_contiguous()
+                 and logits.data_ptr() % 16 == 0 and (logits.shape[-1] * logits.element_size()) % 16 == 0)
+        if not fused:
+            x0, transfer = self.get_transfer_index(logits, temperature, remasking,
+                                                   current_blocks == self.config.mask_id, current_blocks, threshold)
+            committed_rows += transfer.any(dim=1).sum().to(torch.int32)
+            return torch.where(transfer, x0, current_blocks)
+        if temperature == 0:
+            x0, x0_p = ops.argmax_confidence(logits)
+        else:
+            x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
+            _, x0_p = ops.argmax_confidence(logits, picks=x0)
+        out = current_blocks.contiguous().clone()
+        ops.commit_tokens(out, x0.view_as(out).contiguous(), x0_p.view_as(out).contiguous(), committed_rows,
+                          self.config.mask_id, threshold)
+        return out
+
     def get_transfer_index(self, logits, temperature, remasking, mask_index, x, threshold=0.9):
         """Pick the tokens to commit: confidence >= threshold among masked positions, at least one per row."""
         fused = (logits.is_cuda and logits.stride(-1) == 1 and logits.data_ptr() % 16 == 0

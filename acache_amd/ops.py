@@ -269,6 +269,24 @@ def argmax_confidence(logits: torch.Tensor, picks: torch.Tensor | None = None):
     return token.view(logits.shape[:-1]), conf.view(logits.shape[:-1])
 
 
+def commit_tokens(blocks: torch.Tensor, proposal: torch.Tensor, confidence: torch.Tensor,
+                  committed_rows: torch.Tensor, mask_id: int, threshold: float) -> None:
+    """Write the accepted proposals into ``blocks`` (``[n, L]`` int64, in place): positions that hold ``mask_id``
+    and are proposed another token are accepted when their confidence reaches ``threshold``; a row with such
+    positions and none accepted takes its most confident one.  ``committed_rows`` (one int32 on the device) grows
+    by the number of rows that accepted something.  The rule of ``ModelRunner.get_transfer_index`` plus the write
+    of its picks (nano-vdllm/model_runner.py:2297-2314, 2262-2266) in one launch."""
+    assert blocks.is_cuda and blocks.dim() == 2 and blocks.dtype == torch.int64 and blocks.is_contiguous()
+    assert proposal.shape == blocks.shape and proposal.dtype == torch.int64 and proposal.is_contiguous()
+    assert confidence.shape == blocks.shape and confidence.dtype == torch.float32 and confidence.is_contiguous()
+    assert committed_rows.is_cuda and committed_rows.dtype == torch.int32 and committed_rows.numel() == 1
+    lib = _lib.load()
+    with torch.cuda.device(blocks.device):
+        rc = lib.acache_commit_tokens(_ptr(blocks), _ptr(proposal), _ptr(confidence), _ptr(committed_rows),
+                                      blocks.shape[0], blocks.shape[1], int(mask_id), float(threshold), _stream(blocks))
+    _lib.check(rc, "commit_tokens")
+
+
 def swiglu(gate_up: torch.Tensor, hidden: int) -> torch.Tensor:
     """``silu(gate_up[..., :hidden]) * gate_up[..., hidden:]`` of a merged gate / up projection in one pass (the
     MLP activation of the decoder block: ``act(ff_proj(x)) * up_proj(x)``)."""

@@ -282,6 +282,30 @@ int acache_argmax_confidence(
     int64_t R, int64_t V, int64_t row_stride, int32_t dtype, void *stream);
 
 /*
+ * The commit step behind it: write the accepted proposals into the working blocks.
+ *
+ *   for r < n, i < L (blocks, proposal: int64 [n, L]; confidence: fp32 [n, L]; all contiguous):
+ *     committable[r, i] = blocks[r, i] == mask_id && proposal[r, i] != mask_id
+ *     accept[r, i]      = committable[r, i] && confidence[r, i] >= threshold
+ *     a row with committable positions and no accepted one accepts its most confident
+ *     committable position (the first of equals)
+ *     blocks[r, i] = proposal[r, i] where accepted; every other entry is left as it is
+ *   *committed_rows += number of rows that accepted at least one position (atomic; the caller
+ *   compares the counter before and after to learn whether the step made progress)
+ *
+ * Replaces the mask / threshold / forced-pick tensor operations of get_transfer_index and the
+ * write of its picks into the working blocks (nano-vdllm/model_runner.py:2297-2314, 2262-2266)
+ * by one launch, one wave per row.  Differs from the reference in the rule this library's host
+ * documents: a position whose proposal is the mask token itself is never accepted (writing it
+ * would change nothing, and as a forced pick it would repeat the same step for ever).
+ * Confidences are expected to be numbers (a NaN is never accepted by threshold and is forced
+ * only when it is the row's first committable position).
+ */
+int acache_commit_tokens(
+    int64_t *blocks, const int64_t *proposal, const float *confidence, int32_t *committed_rows,
+    int64_t n, int32_t L, int64_t mask_id, float threshold, void *stream);
+
+/*
  * Expand per-request block tables into a flat slot map.
  *
  *   out_slots[cu_k[b] + n] = block_tables[b, n / block_size] * block_size + n % block_size

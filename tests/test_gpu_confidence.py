@@ -74,3 +74,54 @@ def test_argument_errors(device):
     x = torch.randn(4, 50, device=device).to(torch.bfloat16)      # 100-byte rows: not 16-byte aligned
     with pytest.raises(ValueError, match="aligned"):
         ops.argmax_confidence(x)
+
+
+def _commit_rule(blocks, proposal, conf, mask_id, threshold):
+    """The commit rule in tensor operations (the formulation of ModelRunner.get_transfer_index and of the write that
+    follows it): returns the new blocks and the number of rows that committed."""
+    committable = (blocks == mask_id) & (proposal != mask_id)
+    c = torch.where(committable, conf, torch.full_like(conf, -float("inf")))
+    accept = (c >= threshold) & committable
+    stuck = committable.any(dim=1) & ~accept.any(dim=1)
+    forced = torch.zeros_like(accept).scatter_(1, c.argmax(dim=1, keepdim=True), stuck.unsqueeze(1))
+    accept = accept | forced
+    return torch.where(accept, proposal, blocks), int(accept.any(dim=1).sum())
+
+
+def test_commit_tokens_hand_computed(device):
+    M = 9
+    blocks = torch.tensor([[M, M, 5, M],        # one above the threshold
+                           [M, M, M, 7],        # none above: the most confident masked position is forced
+                           [1, 2, 3, 4],        # nothing masked
+                           [M, M, 6, M],        # the most confident proposal is the mask token itself: skipped
+                           [M, M, M, M]], device=device)      # every proposal is the mask token: nothing to commit
+    proposal = torch.tensor([[11, 12, 13, 14], [21, 22, 23, 24], [31, 32, 33, 34], [M, 42, 43, 44], [M, M, M, M]],
+                            device=device)
+    conf = torch.tensor([[0.2, 0.95, 0.99, 0.5], [0.3, 0.6, 0.6, 0.99], [0.9, 0.9, 0.9, 0.9], [0.99, 0.1, 0.99, 0.4],
+                         [0.9, 0.9, 0.9, 0.9]], device=device)
+    counter = torch.zeros(1, dtype=torch.int32, device=device)
+    out = blocks.clone()
+    ops.commit_tokens(out, proposal, conf, counter, M, 0.9)
+    assert out.tolist() == [[M, 12, 5, M], [M, 22, M, 7], [1, 2, 3, 4], [M, M, 6, 44], [M, M, M, M]]
+    assert counter.item() == 3
+    ops.commit_tokens(out, proposal, conf, counter, M, 0.9)   # the counter accumulates; rows 0, 1 and 3 go on
+    assert out.tolist() == [[M, 12, 5, 14], [M, 22, 23, 7], [1, 2, 3, 4], [M, 42, 6, 44], [M, M, M, M]]
+    assert counter.item() == 6
+
+
+@pytest.mark.parametrize("n,L", [(1, 1), (3, 4), (16, 32), (5, 64), (7, 100), (2, 300)])
+def test_commit_tokens_equals_the_tensor_formulation(device, n, L):
+    g = torch.Generator(device=device).manual_seed(n * 1000 + L)
+    M = 63
+    for trial in range(6):
+        blocks = torch.randint(0, 63, (n, L), generator=g, device=device)
+        blocks[torch.rand(n, L, generator=g, device=device) < (0.15 * trial)] = M
+        proposal = torch.randint(0, 64, (n, L), generator=g, device=device)       # some proposals are the mask token
+        conf = torch.rand(n, L, generator=g, device=device)
+        conf = (conf * 8).round() / 8                                           # plenty of ties, also at the maximum
+        threshold = [0.0, 0.5, 0.875, 1.0, 1.5, 0.9][trial]
+        want, rows = _commit_rule(blocks, proposal, conf, M, threshold)
+        counter = torch.zeros(1, dtype=torch.int32, device=device)
+        got = blocks.clone()
+        ops.commit_tokens(got, proposal, conf, counter, M, threshold)
+        assert torch.equal(got, want) and counter.item() == rows
