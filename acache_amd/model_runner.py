@@ -1176,7 +1176,9 @@ class ModelRunner:
     def _commit_from_logits(self, logits, current_blocks, temperature, remasking, threshold, committed_rows):
         """``current_blocks`` with this step's picks written in, by the rule of ``get_transfer_index``.  With
         confidence-based remasking and logits the confidence kernel takes, proposal, confidence and commit are
-        two or three launches; otherwise the tensor formulation.  ``committed_rows`` counts rows that committed."""
+        two or three launches; otherwise the tensor formulation.  ``committed_rows`` counts rows that committed.
+        ``current_blocks`` is the caller's own copy (the result of indexing the working blocks) and may be
+        written in place."""
         fused = (remasking == "low_confidence" and logits.is_cuda and logits.is_contiguous()
                  and logits.data_ptr() % 16 == 0 and (logits.shape[-1] * logits.element_size()) % 16 == 0)
         if not fused:
@@ -1189,7 +1191,7 @@ class ModelRunner:
         else:
             x0 = torch.argmax(add_gumbel_noise(logits, temperature=temperature), dim=-1)
             _, x0_p = ops.argmax_confidence(logits, picks=x0)
-        out = current_blocks.contiguous().clone()
+        out = current_blocks if current_blocks.is_contiguous() else current_blocks.contiguous()
         ops.commit_tokens(out, x0.view_as(out).contiguous(), x0_p.view_as(out).contiguous(), committed_rows,
                           self.config.mask_id, threshold)
         return out
