@@ -86,8 +86,11 @@ void plan_order(const std::vector<int32_t> &costs, int slots, std::vector<int32_
     start[*it] = filled[best_bin[*it]];
     filled[best_bin[*it]] += costs[*it];
   }
-  std::reverse(order.begin(), order.end());
-  std::stable_sort(order.begin(), order.end(), [&](int a, int c) { return start[a] < start[c]; });
+  // units that start together (the first of every bin above all) go out longest first: the dispatch of a
+  // round takes a few microseconds, and the long ones should have them (about 1 us on configs[3])
+  std::stable_sort(order.begin(), order.end(), [&](int a, int c) {
+    return start[a] != start[c] ? start[a] < start[c] : costs[a] > costs[c];
+  });
 }
 
 }  // namespace
