@@ -36,13 +36,13 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, vendor figure
 # A kernel changed after that commit makes its figure stale: tests/test_traffic_constants.py fails when one of
 # the listed sources has a commit after it, and the counters have to be taken again.
 MEASURED_TRAFFIC = {
-    "relocate_32_layers": {"bytes": 18028.3e6, "commit": "8403741",
+    "relocate_32_layers": {"bytes": 18028.3e6, "commit": "b696828",
                            "sources": ["acache_amd/csrc/relocate.hip", "acache_amd/csrc/common.h"]},
-    "relocate_fp32": {"bytes": 1879.1e6, "commit": "8403741",
+    "relocate_fp32": {"bytes": 1879.1e6, "commit": "b696828",
                       "sources": ["acache_amd/csrc/relocate.hip", "acache_amd/csrc/common.h"]},
-    "scatter_28_layers": {"bytes": 332.0e6, "commit": "8403741",
+    "scatter_28_layers": {"bytes": 332.0e6, "commit": "b696828",
                           "sources": ["acache_amd/csrc/scatter.hip", "acache_amd/csrc/common.h"]},
-    "attention": {"bytes": 349.8e6, "commit": "8403741",
+    "attention": {"bytes": 339.4e6, "commit": "b696828",
                   "sources": ["acache_amd/csrc/attn.hip", "acache_amd/csrc/attn_common.h", "acache_amd/csrc/mma.h",
                               "acache_amd/csrc/common.h", "acache_amd/csrc/attn_plan.hip"]},
 }
